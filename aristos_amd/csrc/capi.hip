@@ -1,0 +1,325 @@
+// The C ABI declared in include/kleos_amd.h: lifecycle, forward, bench, inspection.
+//
+// Mirrors the host side of the reference: kleos::initialize / finalize / getRank / setDevice
+// (csrc/include/kleos/bootstrap.cuh:533-588) and kleos::moe::forwardHost / forwardHostBench
+// (csrc/include/kleos/moe/moe.cuh:146-205), for one GPU and expert-parallel degree 1.
+#include <hip/hip_runtime.h>
+
+#include <cstring>
+#include <vector>
+
+#include "common.hpp"
+#include "kernels.hpp"
+
+namespace kleos_amd {
+namespace {
+
+struct Context {
+    kleos_config_t cfg{};
+    int device = 0;
+    int num_cus = 0;
+    hipStream_t stream = nullptr;
+    char* arena = nullptr;          // one allocation holding every library-owned buffer
+    size_t arena_bytes = 0;
+    LayerParams base{};             // configuration + arena pointers; caller buffers filled per call
+    FusedPlan plan{};
+    uint32_t launch_seq = 0;        // forwards issued, any mode (parity selects the live coarse counts)
+    uint32_t fused_seq = 0;         // fused forwards issued (grid-barrier arrival base)
+    int mode = KLEOS_MODE_FUSED;
+    float phase_ms[5] = {0, 0, 0, 0, 0};
+};
+
+Context* g_ctx = nullptr;   // one context per process, like the reference's global state
+
+#define KLEOS_HIP(expr)                                                                         \
+    do {                                                                                        \
+        hipError_t e_ = (expr);                                                                 \
+        if (e_ != hipSuccess)                                                                   \
+            return fail(KLEOS_EHIP, "<%s:%d> %s:\n    %s: %s", __FILE__, __LINE__, #expr,       \
+                        hipGetErrorName(e_), hipGetErrorString(e_));                            \
+    } while (0)
+
+size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+struct ArenaLayout {
+    size_t logits, topk_expert, topk_prob, combine_den, topk_slot, tile_count, super_count,
+        expert_count, slot_token, h1, y, sched, total;
+    size_t zero_begin, zero_end;   // range that must start as zeros
+};
+
+ArenaLayout layout_arena(const kleos_config_t& c, uint32_t n_tiles, uint32_t n_super) {
+    ArenaLayout L{};
+    size_t off = 0;
+    auto take = [&](size_t bytes) { size_t o = off; off = align_up(off + bytes, 256); return o; };
+    const size_t S = c.S, E = c.E, k = c.k, R = c.cap_rows;
+    // counters first: they are the part cleared at initialisation
+    L.zero_begin = off;
+    L.super_count = take(2 * size_t(n_super) * E * 4);
+    L.sched = take(sched_words(c.E, c.cap_rows) * 4);
+    L.expert_count = take(E * 4);
+    L.zero_end = off;
+    L.logits = take(S * E * 4);
+    L.topk_expert = take(S * k * 4);
+    L.topk_prob = take(S * k * 4);
+    L.combine_den = take(S * 4);
+    L.topk_slot = take(S * k * 4);
+    L.tile_count = take(size_t(n_tiles) * E * 4);
+    L.slot_token = take(E * R * 4);
+    L.h1 = take(E * R * size_t(c.I) * c.elem_bytes);
+    L.y = take(E * R * size_t(c.H) * c.elem_bytes);
+    L.total = off;
+    return L;
+}
+
+int require_ctx(const char* who) {
+    if (!g_ctx) return fail(KLEOS_ESTATE, "%s: Not initialized!", who);
+    return KLEOS_OK;
+}
+
+LayerParams bind(const Context& c, const void* iP, void* oP) {
+    LayerParams p = c.base;
+    const size_t eb = c.cfg.elem_bytes;
+    const char* in = static_cast<const char*>(iP);
+    char* out = static_cast<char*>(oP);
+    // moe.cuh:92-98
+    p.x = in + c.cfg.off_x * eb;
+    p.wg = in + c.cfg.off_gate_w * eb;
+    p.w_up = in + c.cfg.off_w_up * eb;
+    p.w_down = in + c.cfg.off_w_down * eb;
+    p.b_up = in + c.cfg.off_b_up * eb;
+    p.b_down = in + c.cfg.off_b_down * eb;
+    p.gate_out = out + c.cfg.off_gate_out * eb;
+    p.moe_out = out + c.cfg.off_moe_out * eb;
+    return p;
+}
+
+// Enqueues one forward. When ev is non-null (phased mode) it receives 6 recorded events that
+// bracket the five phases.
+int enqueue_forward(Context& c, const void* iP, void* oP, hipEvent_t* ev) {
+    if (!iP || !oP) return fail(KLEOS_EINVAL, "forward: null buffer");
+    if ((reinterpret_cast<uintptr_t>(iP) | reinterpret_cast<uintptr_t>(oP)) & 15u)
+        return fail(KLEOS_EINVAL, "forward: iP and oP must be 16-byte aligned");
+    LayerParams p = bind(c, iP, oP);
+    p.epoch = c.launch_seq++;
+    const int dt = int(c.cfg.torch_dtype);
+    if (c.mode == KLEOS_MODE_FUSED) {
+        KLEOS_HIP(launch_fused(p, c.plan, c.fused_seq++, c.stream));
+        return KLEOS_OK;
+    }
+    if (ev) KLEOS_HIP(hipEventRecord(ev[0], c.stream));
+    KLEOS_HIP(launch_gate(p, dt, c.stream));
+    if (ev) KLEOS_HIP(hipEventRecord(ev[1], c.stream));
+    KLEOS_HIP(launch_slots(p, c.stream));
+    if (ev) KLEOS_HIP(hipEventRecord(ev[2], c.stream));
+    KLEOS_HIP(launch_expert_gemm(p, dt, 0, c.stream));
+    if (ev) KLEOS_HIP(hipEventRecord(ev[3], c.stream));
+    KLEOS_HIP(launch_expert_gemm(p, dt, 1, c.stream));
+    if (ev) KLEOS_HIP(hipEventRecord(ev[4], c.stream));
+    KLEOS_HIP(launch_combine(p, dt, c.stream));
+    if (ev) KLEOS_HIP(hipEventRecord(ev[5], c.stream));
+    return KLEOS_OK;
+}
+
+}  // namespace
+}  // namespace kleos_amd
+
+using namespace kleos_amd;
+
+extern "C" int kleos_initialize_cfg(const kleos_config_t* user_cfg) {
+    if (!user_cfg) return fail(KLEOS_EINVAL, "kleos_initialize_cfg: null config");
+    if (g_ctx) return fail(KLEOS_ESTATE, "Already Initialized");   // bootstrap.cuh:537
+    kleos_config_t cfg = *user_cfg;
+    if (int rc = kleos_config_derive(&cfg)) return rc;
+    if (const char* why = unsupported_reason(cfg.E, cfg.k)) return fail(KLEOS_EUNSUPPORTED, "%s", why);
+
+    Context* c = new Context();
+    c->cfg = cfg;
+    auto bail = [&](int rc) {
+        if (c->arena) (void)hipFree(c->arena);
+        if (c->stream) (void)hipStreamDestroy(c->stream);
+        delete c;
+        return rc;
+    };
+#define KLEOS_HIP_BAIL(expr)                                                                    \
+    do {                                                                                        \
+        hipError_t e_ = (expr);                                                                 \
+        if (e_ != hipSuccess)                                                                   \
+            return bail(fail(KLEOS_EHIP, "<%s:%d> %s:\n    %s: %s", __FILE__, __LINE__, #expr,  \
+                             hipGetErrorName(e_), hipGetErrorString(e_)));                      \
+    } while (0)
+    KLEOS_HIP_BAIL(hipGetDevice(&c->device));
+    hipDeviceProp_t prop;
+    KLEOS_HIP_BAIL(hipGetDeviceProperties(&prop, c->device));
+    c->num_cus = prop.multiProcessorCount;
+    if (std::strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return bail(fail(KLEOS_EUNSUPPORTED, "device '%s' is not gfx950: this library is built for MI355X only",
+                         prop.gcnArchName));
+    // default priority, non-blocking: the analogue of the reference's cudaStreamPerThread (types.cuh:1013)
+    KLEOS_HIP_BAIL(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
+
+    LayerParams& p = c->base;
+    p.S = cfg.S; p.H = cfg.H; p.I = cfg.I; p.E = cfg.E; p.k = cfg.k; p.PX = cfg.PX;
+    p.EC = cfg.EC; p.cap_rows = cfg.cap_rows; p.act = cfg.hidden_act;
+    p.n_gate_tiles = cfg.S / kGateTileTokens;
+    p.n_super = (p.n_gate_tiles + kSuperTiles - 1) / kSuperTiles;
+    const ArenaLayout L = layout_arena(cfg, p.n_gate_tiles, p.n_super);
+    KLEOS_HIP_BAIL(hipMalloc(reinterpret_cast<void**>(&c->arena), L.total));
+    c->arena_bytes = L.total;
+    KLEOS_HIP_BAIL(hipMemsetAsync(c->arena + L.zero_begin, 0, L.zero_end - L.zero_begin, c->stream));
+    KLEOS_HIP_BAIL(hipStreamSynchronize(c->stream));
+    char* a = c->arena;
+    p.logits = reinterpret_cast<float*>(a + L.logits);
+    p.topk_expert = reinterpret_cast<int32_t*>(a + L.topk_expert);
+    p.topk_prob = reinterpret_cast<float*>(a + L.topk_prob);
+    p.combine_den = reinterpret_cast<float*>(a + L.combine_den);
+    p.topk_slot = reinterpret_cast<int32_t*>(a + L.topk_slot);
+    p.tile_count = reinterpret_cast<uint32_t*>(a + L.tile_count);
+    p.super_count = reinterpret_cast<uint32_t*>(a + L.super_count);
+    p.expert_count = reinterpret_cast<uint32_t*>(a + L.expert_count);
+    p.slot_token = reinterpret_cast<int32_t*>(a + L.slot_token);
+    p.h1 = a + L.h1;
+    p.y = a + L.y;
+    p.sched = reinterpret_cast<uint32_t*>(a + L.sched);
+    KLEOS_HIP_BAIL(plan_fused(p, int(cfg.torch_dtype), c->num_cus, &c->plan));
+#undef KLEOS_HIP_BAIL
+    g_ctx = c;
+    return KLEOS_OK;
+}
+
+extern "C" int kleos_initialize(const char* config_json_path) {
+    if (g_ctx) return fail(KLEOS_ESTATE, "Already Initialized");
+    kleos_config_t cfg;
+    if (int rc = kleos_config_parse_file(config_json_path, &cfg)) return rc;
+    return kleos_initialize_cfg(&cfg);
+}
+
+extern "C" int kleos_finalize(void) {
+    if (int rc = require_ctx("kleos_finalize")) return rc;
+    Context* c = g_ctx;
+    g_ctx = nullptr;   // bootstrap.cuh:567: isInitialized = false first
+    hipError_t e1 = hipSetDevice(c->device);
+    hipError_t e2 = hipStreamSynchronize(c->stream);
+    hipError_t e3 = hipFree(c->arena);
+    hipError_t e4 = hipStreamDestroy(c->stream);
+    delete c;
+    for (hipError_t e : {e1, e2, e3, e4})
+        if (e != hipSuccess) return fail(KLEOS_EHIP, "kleos_finalize: %s: %s", hipGetErrorName(e), hipGetErrorString(e));
+    return KLEOS_OK;
+}
+
+extern "C" int kleos_is_initialized(void) { return g_ctx != nullptr; }
+
+extern "C" int kleos_get_rank(void) {
+    if (!g_ctx) { (void)fail(KLEOS_ESTATE, "kleos_get_rank: Not initialized!"); return -1; }
+    return 0;
+}
+
+extern "C" int kleos_set_device(void) {
+    if (int rc = require_ctx("kleos_set_device")) return rc;
+    KLEOS_HIP(hipSetDevice(g_ctx->device));
+    return KLEOS_OK;
+}
+
+extern "C" int kleos_get_config(kleos_config_t* cfg) {
+    if (int rc = require_ctx("kleos_get_config")) return rc;
+    if (!cfg) return fail(KLEOS_EINVAL, "kleos_get_config: null argument");
+    *cfg = g_ctx->cfg;
+    return KLEOS_OK;
+}
+
+extern "C" int kleos_set_mode(int mode) {
+    if (int rc = require_ctx("kleos_set_mode")) return rc;
+    if (mode != KLEOS_MODE_FUSED && mode != KLEOS_MODE_PHASED) return fail(KLEOS_EINVAL, "kleos_set_mode: unknown mode %d", mode);
+    g_ctx->mode = mode;
+    return KLEOS_OK;
+}
+
+extern "C" int kleos_get_mode(void) { return g_ctx ? g_ctx->mode : -1; }
+
+extern "C" int kleos_moe_forward(const void* iP, void* oP) {
+    if (int rc = require_ctx("kleos_moe_forward")) return rc;
+    KLEOS_HIP(hipSetDevice(g_ctx->device));   // moe.cuh:192
+    return enqueue_forward(*g_ctx, iP, oP, nullptr);
+}
+
+extern "C" int kleos_moe_forward_bench(const void* iP, void* oP, uint32_t skip, uint32_t trials,
+                                       float* ms_per_launch) {
+    if (int rc = require_ctx("kleos_moe_forward_bench")) return rc;
+    if (!ms_per_launch || trials == 0) return fail(KLEOS_EINVAL, "kleos_moe_forward_bench: need trials > 0 and a result pointer");
+    Context& c = *g_ctx;
+    KLEOS_HIP(hipSetDevice(c.device));
+    for (uint32_t i = 0; i < skip; ++i)
+        if (int rc = enqueue_forward(c, iP, oP, nullptr)) return rc;
+    const bool phased = c.mode == KLEOS_MODE_PHASED;
+    hipEvent_t start, stop;
+    KLEOS_HIP(hipEventCreate(&start));
+    KLEOS_HIP(hipEventCreate(&stop));
+    std::vector<hipEvent_t> ev;
+    if (phased) {
+        ev.resize(size_t(trials) * 6);
+        for (auto& e : ev) KLEOS_HIP(hipEventCreate(&e));
+    }
+    int rc = KLEOS_OK;
+    KLEOS_HIP(hipEventRecord(start, c.stream));                       // moe.cuh:166
+    for (uint32_t i = 0; i < trials && rc == KLEOS_OK; ++i)
+        rc = enqueue_forward(c, iP, oP, phased ? &ev[size_t(i) * 6] : nullptr);
+    if (rc == KLEOS_OK) {
+        KLEOS_HIP(hipEventRecord(stop, c.stream));                    // moe.cuh:178
+        KLEOS_HIP(hipStreamSynchronize(c.stream));
+        float ms = 0.f;
+        KLEOS_HIP(hipEventElapsedTime(&ms, start, stop));
+        *ms_per_launch = ms / float(trials);                          // moe.cuh:181
+        for (float& v : c.phase_ms) v = 0.f;
+        if (phased) {
+            for (uint32_t i = 0; i < trials; ++i)
+                for (int ph = 0; ph < 5; ++ph) {
+                    float t = 0.f;
+                    KLEOS_HIP(hipEventElapsedTime(&t, ev[size_t(i) * 6 + ph], ev[size_t(i) * 6 + ph + 1]));
+                    c.phase_ms[ph] += t / float(trials);
+                }
+        }
+    } else {
+        (void)hipStreamSynchronize(c.stream);
+    }
+    (void)hipEventDestroy(start);
+    (void)hipEventDestroy(stop);
+    for (auto& e : ev) (void)hipEventDestroy(e);
+    return rc;
+}
+
+extern "C" int kleos_stream_synchronize(void) {
+    if (int rc = require_ctx("kleos_stream_synchronize")) return rc;
+    KLEOS_HIP(hipStreamSynchronize(g_ctx->stream));
+    return KLEOS_OK;
+}
+
+extern "C" void* kleos_stream(void) { return g_ctx ? static_cast<void*>(g_ctx->stream) : nullptr; }
+
+extern "C" int kleos_moe_debug_views(kleos_debug_views_t* v) {
+    if (int rc = require_ctx("kleos_moe_debug_views")) return rc;
+    if (!v) return fail(KLEOS_EINVAL, "kleos_moe_debug_views: null argument");
+    const LayerParams& p = g_ctx->base;
+    v->logits = p.logits;
+    v->topk_expert = p.topk_expert;
+    v->topk_prob = p.topk_prob;
+    v->combine_den = p.combine_den;
+    v->topk_slot = p.topk_slot;
+    v->expert_count = p.expert_count;
+    v->slot_token = p.slot_token;
+    return KLEOS_OK;
+}
+
+extern "C" int kleos_debug_copy_to_host(void* host_dst, const void* device_src, size_t bytes) {
+    if (int rc = require_ctx("kleos_debug_copy_to_host")) return rc;
+    if (!host_dst || !device_src) return fail(KLEOS_EINVAL, "kleos_debug_copy_to_host: null argument");
+    KLEOS_HIP(hipStreamSynchronize(g_ctx->stream));
+    KLEOS_HIP(hipMemcpy(host_dst, device_src, bytes, hipMemcpyDeviceToHost));
+    return KLEOS_OK;
+}
+
+extern "C" int kleos_phase_times(float ms[5]) {
+    if (int rc = require_ctx("kleos_phase_times")) return rc;
+    if (!ms) return fail(KLEOS_EINVAL, "kleos_phase_times: null argument");
+    for (int i = 0; i < 5; ++i) ms[i] = g_ctx->phase_ms[i];
+    return KLEOS_OK;
+}

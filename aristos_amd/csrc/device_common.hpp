@@ -1,0 +1,80 @@
+// Small device-side vocabulary shared by the kernels: vector types, Element conversions,
+// matrix-core wrappers, scoped atomics.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+#include "layer.hpp"
+
+namespace kleos_amd {
+
+typedef __bf16 bf16_t;
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int kWave = 64;
+
+__device__ __forceinline__ float elem_to_float(bf16_t v) { return static_cast<float>(v); }
+__device__ __forceinline__ float elem_to_float(float v) { return v; }
+
+// fp32 -> Element, round to nearest even (cutlass::NumericConverter in the reference).
+template <typename T>
+__device__ __forceinline__ T float_to_elem(float v);
+template <>
+__device__ __forceinline__ float float_to_elem<float>(float v) { return v; }
+template <>
+__device__ __forceinline__ bf16_t float_to_elem<bf16_t>(float v) { return static_cast<bf16_t>(v); }
+
+__device__ __forceinline__ u32x4 load16(const void* p) { return *reinterpret_cast<const u32x4*>(p); }
+__device__ __forceinline__ void store16(void* p, u32x4 v) { *reinterpret_cast<u32x4*>(p) = v; }
+
+// Activations of the reference (types.cuh:151-159): 0 = ReLU<float>, 1 = erf GELU<float>.
+template <int ACT>
+__device__ __forceinline__ float activate(float v) {
+    if constexpr (ACT == 0) return v > 0.0f ? v : 0.0f;
+    else if constexpr (ACT == 1) return 0.5f * v * (1.0f + erff(v * 0.70710678118654752440f));
+    else return v;
+}
+
+// One matrix-core step on 16 bytes of K per lane from each operand, 16x16 output.
+//   a: lane l holds row  (l % 16) of the 16-row operand, K-chunk (l / 16)
+//   b: lane l holds col  (l % 16) of the 16-col operand, K-chunk (l / 16)
+//   acc[v]: element (row 4*(l/16)+v, col l%16)
+// For bf16 one instruction consumes 32 values of K; for fp32 four instructions consume 16.
+__device__ __forceinline__ f32x4 mma16_step(u32x4 a, u32x4 b, f32x4 acc, bf16_t) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a),
+                                                   __builtin_bit_cast(bf16x8, b), acc, 0, 0, 0);
+}
+__device__ __forceinline__ f32x4 mma16_step(u32x4 a, u32x4 b, f32x4 acc, float) {
+    f32x4 fa = __builtin_bit_cast(f32x4, a), fb = __builtin_bit_cast(f32x4, b);
+    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[0], fb[0], acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[1], fb[1], acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[2], fb[2], acc, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[3], fb[3], acc, 0, 0, 0);
+    return acc;
+}
+
+// Device-scope (agent) atomics: the scheduler counters are shared by workgroups on different
+// XCDs, whose L2 caches are not coherent with each other for ordinary loads and stores.
+__device__ __forceinline__ uint32_t atomic_add_agent(uint32_t* p, uint32_t v) {
+    return __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ uint32_t atomic_add_release(uint32_t* p, uint32_t v) {
+    return __hip_atomic_fetch_add(p, v, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ uint32_t atomic_load_acquire(const uint32_t* p) {
+    return __hip_atomic_load(p, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ uint32_t atomic_load_relaxed(const uint32_t* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void atomic_store_relaxed(uint32_t* p, uint32_t v) {
+    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+}  // namespace kleos_amd

@@ -1,0 +1,34 @@
+// Host-callable launchers of the layer's kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include "layer.hpp"
+
+namespace kleos_amd {
+
+// Number of uint32 scheduler words the persistent kernel needs for a layer with these sizes.
+size_t sched_words(uint32_t E, uint32_t cap_rows);
+
+// Phase launchers (KLEOS_MODE_PHASED). dtype: 0 fp32, 2 bf16.
+hipError_t launch_gate(const LayerParams& p, int dtype, hipStream_t s);
+hipError_t launch_slots(const LayerParams& p, hipStream_t s);
+hipError_t launch_expert_gemm(const LayerParams& p, int dtype, int kind /*0 up, 1 down*/, hipStream_t s);
+hipError_t launch_combine(const LayerParams& p, int dtype, hipStream_t s);
+
+// The whole layer as one persistent launch (KLEOS_MODE_FUSED). The plan fixes the grid (every
+// workgroup resident at once), the LDS size and the scheduler constants for a configuration.
+struct FusedPlan {
+    const void* kernel = nullptr;
+    uint32_t nwg = 0;
+    size_t smem = 0;
+    uint32_t mt_max = 0;   // row blocks per expert at full capacity
+    uint32_t lag = 0;      // experts between an up-projection segment and its down-projection segment
+};
+hipError_t plan_fused(const LayerParams& p, int dtype, int num_cus, FusedPlan* plan);
+// fused_seq: number of fused launches already issued on this scheduler arena.
+hipError_t launch_fused(const LayerParams& p, const FusedPlan& plan, uint32_t fused_seq, hipStream_t s);
+
+// Why a configuration cannot run, or nullptr when it can.
+const char* unsupported_reason(uint32_t E, uint32_t k);
+
+}  // namespace kleos_amd

@@ -1,0 +1,52 @@
+// Device-visible description of one MoE layer invocation: configuration, the caller's packed
+// buffers sliced into their parts, and the library-owned arenas. Passed by value to every kernel.
+#pragma once
+#include <cstdint>
+
+namespace kleos_amd {
+
+constexpr int kGateTileTokens = 16;   // tokens per gate tile (one MFMA column block)
+constexpr int kSuperTiles = 32;       // gate tiles per coarse count row (512 tokens)
+constexpr int kMaxGateGroups = 16;    // 16 experts per group -> gate handles E <= 256
+
+// Work item of the expert phase: one output tile of the up- or down-projection.
+struct TileTask {
+    uint16_t expert;
+    uint16_t kind;      // 0 up-projection, 1 down-projection
+    uint32_t row0;      // first slot (row inside the expert's buffer)
+    uint32_t col0;      // first output column
+};
+
+struct LayerParams {
+    // ---- configuration (derived as the reference's struct ACC, types.cuh:471-507)
+    uint32_t S, H, I, E, k, PX, EC, cap_rows, act;
+    uint32_t n_gate_tiles;    // S / 16
+    uint32_t n_super;         // ceil(n_gate_tiles / 32)
+    // ---- caller buffers, sliced as moe.cuh:92-98
+    const void* x;            // [S, H]
+    const void* wg;           // [PX, H]
+    const void* w_up;         // [E][I, H]
+    const void* w_down;       // [E][H, I]
+    const void* b_up;         // [E][I]
+    const void* b_down;       // [E][H]
+    void* gate_out;           // [S, PX]
+    void* moe_out;            // [S, H]
+    // ---- routing arenas (reference: Bookkeeping tP/eC, types.cuh:836-842)
+    float* logits;            // [S, E]
+    int32_t* topk_expert;     // [S, k]
+    float* topk_prob;         // [S, k]
+    float* combine_den;       // [S]
+    int32_t* topk_slot;       // [S, k]  in-tile rank after the gate, final slot or -1 after slotting
+    uint32_t* tile_count;     // [n_gate_tiles, E]   tokens of each 16-token tile routed to e
+    uint32_t* super_count;    // [2][n_super, E]     the same summed over 32 tiles; two epochs
+    uint32_t* expert_count;   // [E]
+    int32_t* slot_token;      // [E, cap_rows]
+    // ---- intermediate activations (reference: xM buffer, types.cuh:976-982)
+    void* h1;                 // [E][cap_rows, I]
+    void* y;                  // [E][cap_rows, H]
+    // ---- scheduler state of the persistent kernel
+    uint32_t* sched;          // counters, see scheduler section of moe_kernels.hip
+    uint32_t epoch;           // launch parity, selects the live half of double-buffered counters
+};
+
+}  // namespace kleos_amd

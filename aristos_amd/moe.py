@@ -1,0 +1,71 @@
+"""Host API of the MoE forward, named after the reference's kleos::moe functions
+(csrc/include/kleos/moe/moe.cuh:146-205). Buffers are device pointers (ints) or objects with a
+``data_ptr()`` method (torch tensors); nothing here touches their contents on the host."""
+from __future__ import annotations
+
+import ctypes as C
+
+import numpy as np
+
+from . import _capi
+
+
+def _ptr(buf) -> int:
+    if isinstance(buf, int):
+        return buf
+    if hasattr(buf, "data_ptr"):
+        return int(buf.data_ptr())
+    raise TypeError(f"expected a device pointer or tensor, got {type(buf)!r}")
+
+
+def forward_host(iP, oP) -> None:
+    """kleos::moe::forwardHost(iP, oP) (moe.cuh:186-205): enqueue one forward on the library stream."""
+    _capi.check(_capi.lib().kleos_moe_forward(_ptr(iP), _ptr(oP)))
+
+
+def forward_host_bench(iP, oP, skip: int = 32, trials: int = 32) -> float:
+    """kleos::moe::forwardHostBench<skip, trials>(iP, oP, ms) (moe.cuh:146-184): mean milliseconds per
+    launch over `trials` launches after `skip` warm-ups. The defaults are the reference driver's
+    (csrc/main.cu:68)."""
+    ms = C.c_float(0.0)
+    _capi.check(_capi.lib().kleos_moe_forward_bench(_ptr(iP), _ptr(oP), skip, trials, C.byref(ms)))
+    return float(ms.value)
+
+
+def stream_synchronize() -> None:
+    _capi.check(_capi.lib().kleos_stream_synchronize())
+
+
+def set_mode(mode: int) -> None:
+    """MODE_FUSED (one persistent launch, default) or MODE_PHASED (one launch per phase)."""
+    _capi.check(_capi.lib().kleos_set_mode(int(mode)))
+
+
+def phase_times() -> dict:
+    """Per-phase milliseconds of the last phased forward_host_bench."""
+    arr = (C.c_float * 5)()
+    _capi.check(_capi.lib().kleos_phase_times(arr))
+    return dict(zip(("gate", "slots", "up", "down", "combine"), (float(v) for v in arr)))
+
+
+def debug_views(derived) -> dict:
+    """Copies the routing state of the most recent forward to host numpy arrays. Synchronises."""
+    lib = _capi.lib()
+    v = _capi.DebugViewsStruct()
+    _capi.check(lib.kleos_moe_debug_views(C.byref(v)))
+    S, E, k, R = derived.S, derived.E, derived.k, derived.cap_rows
+    spec = {
+        "logits": (v.logits, (S, E), np.float32),
+        "topk_expert": (v.topk_expert, (S, k), np.int32),
+        "topk_prob": (v.topk_prob, (S, k), np.float32),
+        "combine_den": (v.combine_den, (S,), np.float32),
+        "topk_slot": (v.topk_slot, (S, k), np.int32),
+        "expert_count": (v.expert_count, (E,), np.uint32),
+        "slot_token": (v.slot_token, (E, R), np.int32),
+    }
+    out = {}
+    for name, (ptr, shape, dt) in spec.items():
+        host = np.empty(shape, dtype=dt)
+        _capi.check(lib.kleos_debug_copy_to_host(host.ctypes.data, ptr, host.nbytes))
+        out[name] = host
+    return out

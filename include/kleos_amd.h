@@ -1,0 +1,174 @@
+/*
+ * kleos_amd.h — C ABI of the MI355X-native fused MoE forward.
+ *
+ * This is the drop-in boundary for the single-GPU (expert-parallel degree 1) MoE layer forward of
+ * Kleos/FlashDMoE. Every entry point names the reference interface it replaces. All pointers are
+ * plain host or device pointers, sizes are in bytes or elements as stated; no C++ or framework
+ * types cross this boundary. Every function returning int returns 0 on success and a non-zero
+ * KLEOS_E* code on failure; the text of the last failure is available from kleos_last_error().
+ *
+ * Threading: like the reference (process-global isInitialized / hostBookkeeping / seqBit,
+ * reference csrc/include/kleos/types.cuh:440,1011-1012) the library holds ONE context per process.
+ * Calls are not re-entrant; forwards issued back-to-back on the library stream are ordered.
+ */
+#ifndef KLEOS_AMD_H
+#define KLEOS_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- error codes --------------------------------------------------------------------------- */
+enum {
+    KLEOS_OK = 0,
+    KLEOS_EINVAL = 1,      /* bad argument / invalid configuration value          */
+    KLEOS_ESTATE = 2,      /* "Not initialized!" / "Already Initialized"           */
+    KLEOS_EUNSUPPORTED = 3,/* valid reference config this build does not implement */
+    KLEOS_EHIP = 4,        /* a HIP runtime call failed                            */
+    KLEOS_EIO = 5,         /* config file could not be read                        */
+    KLEOS_EPARSE = 6       /* config JSON malformed or a required key is missing   */
+};
+
+/* ---- configuration -------------------------------------------------------------------------- */
+/* torch_dtype enumeration of the reference (csrc/kleos_config.schema.json:64-68). */
+enum { KLEOS_DTYPE_FP32 = 0, KLEOS_DTYPE_TF32 = 1, KLEOS_DTYPE_BF16 = 2, KLEOS_DTYPE_FP16 = 3 };
+/* hidden_act enumeration of the reference (csrc/kleos_config.schema.json:29-33). */
+enum { KLEOS_ACT_RELU = 0, KLEOS_ACT_GELU = 1 };
+
+/*
+ * The keys of kleos_config.json (reference csrc/kleos_config.schema.json:5-72) followed by the
+ * constants the reference derives from them at compile time in struct ACC
+ * (csrc/include/kleos/types.cuh:471-507). The reference consumes the JSON at CMake configure time
+ * (csrc/CMakeLists.txt:186-252); here it is read at run time.
+ */
+typedef struct kleos_config {
+    /* -- JSON keys -- */
+    double   capacity_factor;   /* reference: integer >= 1; this build also takes real values   */
+    uint32_t drop_tokens;       /* 0 | 1                                                         */
+    uint32_t expert_top_k;
+    uint32_t global_batch;      /* parsed, unused: feeds only the reference's placement models   */
+    uint32_t is_training;       /* 0 | 1                                                         */
+    uint32_t hidden_act;        /* KLEOS_ACT_*                                                   */
+    uint32_t hidden_size;       /* H                                                             */
+    uint32_t intermediate_size; /* I  ("P" in the reference)                                     */
+    uint32_t mini_batch;
+    uint32_t moe_frequency;     /* parsed, unused                                                */
+    uint32_t num_experts;       /* E                                                             */
+    uint32_t num_layers;        /* parsed, unused                                                */
+    uint32_t sequence_len;
+    uint32_t torch_dtype;       /* KLEOS_DTYPE_*                                                 */
+    uint32_t vocab_size;        /* parsed, unused                                                */
+    /* -- derived (types.cuh:471-507) -- */
+    uint32_t S;                 /* tokens = sequence_len * mini_batch              (:471)        */
+    uint32_t H, I, E, k;
+    uint32_t PX;                /* experts padded to a multiple of 64              (:481)        */
+    uint32_t EC;                /* expert capacity                                 (:498-499)    */
+    uint32_t pEC;               /* EC padded to a multiple of 128                  (:500)        */
+    uint32_t cap_rows;          /* min(pEC, S): row stride of every per-expert buffer. An expert
+                                 * never holds more than S tokens, so without token dropping
+                                 * (EC = S*cf*k) the arenas are sized by S instead.              */
+    uint32_t elem_bytes;        /* sizeof(Element): 4 (fp32) or 2 (bf16)                         */
+    /* Element offsets into the packed input buffer iP (csrc/include/kleos/moe/moe.cuh:92-96,
+     * csrc/main.cu:23-28) and the packed output buffer oP (moe.cuh:97-98). */
+    uint64_t off_x, off_gate_w, off_w_up, off_w_down, off_b_up, off_b_down, in_elems;
+    uint64_t off_gate_out, off_moe_out, out_elems;
+} kleos_config_t;
+
+/* Parse a kleos_config.json text / file into cfg (keys only, no derivation, no validation beyond
+ * JSON well-formedness and presence of the schema's required keys). */
+int kleos_config_parse_string(const char* json_text, kleos_config_t* cfg);
+int kleos_config_parse_file(const char* path, kleos_config_t* cfg);
+/* Fill cfg with the shipped defaults of the reference (csrc/kleos_config.json:1-17) except
+ * torch_dtype = bf16. */
+void kleos_config_defaults(kleos_config_t* cfg);
+/* Validate the keys and fill the derived fields. Enforces the reference's static_asserts
+ * (csrc/include/kleos/bootstrap.cuh:542-545; types.cuh:479,496-497): S % 128 == 0, I % 64 == 0,
+ * H % 64 == 0, k <= E, E <= 65535, capacity_factor >= 1. tf32 and fp16 yield KLEOS_EUNSUPPORTED. */
+int kleos_config_derive(kleos_config_t* cfg);
+
+/* ---- lifecycle ------------------------------------------------------------------------------ */
+/* Replaces kleos::initialize() (csrc/include/kleos/bootstrap.cuh:533-547): validates the config,
+ * selects the device, creates the library stream and allocates every scratch arena (routing
+ * tables, intermediate activations, scheduler counters) the forward needs, as the reference's
+ * Bookkeeping arenas are (bootstrap.cuh:377-391). Fails with KLEOS_ESTATE "Already Initialized". */
+int kleos_initialize(const char* config_json_path);
+int kleos_initialize_cfg(const kleos_config_t* cfg);
+/* Replaces kleos::finalize() (bootstrap.cuh:562-588): drains the stream, frees every arena. */
+int kleos_finalize(void);
+int kleos_is_initialized(void);
+/* Replaces kleos::getRank() (bootstrap.cuh:556-559): always 0 (expert-parallel degree 1).
+ * Returns -1 when not initialised. */
+int kleos_get_rank(void);
+/* Replaces kleos::setDevice() (bootstrap.cuh:550-553): makes the library's GPU current. */
+int kleos_set_device(void);
+/* Copy of the active configuration (derived fields filled). */
+int kleos_get_config(kleos_config_t* cfg);
+
+/* ---- forward -------------------------------------------------------------------------------- */
+/*
+ * Replaces kleos::moe::forwardHost(iP, oP) (csrc/include/kleos/moe/moe.cuh:186-205).
+ * iP: device pointer, packed Elements  x[S,H] | Wg[PX,H] | Wup[E][I,H] | Wdown[E][H,I] | bup[E][I] | bdown[E][H]
+ * oP: device pointer, packed Elements  gateOut[S,PX] | moeOut[S,H]
+ * Asynchronous on the library stream (the reference launches on kleosStream, types.cuh:1013); the
+ * output is valid after kleos_stream_synchronize(). No host-side reset is needed between calls.
+ * E == 1 runs the dense FFN (moe.cuh:197-204).
+ */
+int kleos_moe_forward(const void* iP, void* oP);
+/*
+ * Replaces kleos::moe::forwardHostBench<skip,trials>(iP, oP, ms) (moe.cuh:146-184): `skip` untimed
+ * launches, then `trials` launches bracketed by events on the library stream; *ms_per_launch is the
+ * mean. Synchronises the stream before returning.
+ */
+int kleos_moe_forward_bench(const void* iP, void* oP, uint32_t skip, uint32_t trials,
+                            float* ms_per_launch);
+/* Blocks until everything queued on the library stream has finished
+ * (cudaStreamSynchronize(kleosStream) in the reference's callers, csrc/main.cu:64-70). */
+int kleos_stream_synchronize(void);
+/* The library stream as an opaque hipStream_t, for callers that want to order their own work
+ * against it. NULL when not initialised. */
+void* kleos_stream(void);
+
+/* Which implementation kleos_moe_forward runs. 0 = one persistent launch with the in-kernel tile
+ * scheduler (default); 1 = the same device functions as a sequence of separate launches, one per
+ * phase (used to time phases in isolation). */
+enum { KLEOS_MODE_FUSED = 0, KLEOS_MODE_PHASED = 1 };
+int kleos_set_mode(int mode);
+int kleos_get_mode(void);
+
+/* ---- inspection (no counterpart in the reference, which exposes only gateOut and moeOut) ---- */
+/*
+ * Device pointers to the routing state left by the most recent forward, for parity checks of the
+ * routing against fp32 logits. The arrays live in library-owned arenas and are overwritten by the
+ * next forward; copy them out after kleos_stream_synchronize().
+ */
+typedef struct kleos_debug_views {
+    const float*    logits;       /* [S, E]  fp32 gate logits (before softmax)                        */
+    const int32_t*  topk_expert;  /* [S, k]  selected experts in selection order (best first)        */
+    const float*    topk_prob;    /* [S, k]  fp32 softmax probability of each selected expert        */
+    const float*    combine_den;  /* [S]     sum of the k selected probabilities (reference "mCw")   */
+    const int32_t*  topk_slot;    /* [S, k]  slot inside the expert's buffer, or -1 when dropped     */
+    const uint32_t* expert_count; /* [E]     tokens routed to each expert, dropped ones included     */
+    const int32_t*  slot_token;   /* [E, cap_rows] token held by each slot (valid for slot < min(count,EC)) */
+} kleos_debug_views_t;
+int kleos_moe_debug_views(kleos_debug_views_t* views);
+/* Drains the library stream, then copies `bytes` from a device pointer (one of the views above, or
+ * any device buffer) into host memory. A convenience for callers without a HIP runtime binding. */
+int kleos_debug_copy_to_host(void* host_dst, const void* device_src, size_t bytes);
+
+/* Per-phase device time of the most recent kleos_moe_forward_bench in KLEOS_MODE_PHASED, in
+ * milliseconds per launch: [0] gate, [1] slotting, [2] up-projection, [3] down-projection,
+ * [4] combine. Zero-filled in fused mode. */
+int kleos_phase_times(float ms[5]);
+
+/* ---- errors --------------------------------------------------------------------------------- */
+/* Replaces the KLEOS_CHECK_CUDA / KLEOS_ASSERT message conventions (csrc/include/kleos/debug.cuh:
+ * 19-43), which print and exit; the C ABI records the message and returns a code instead. */
+const char* kleos_last_error(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* KLEOS_AMD_H */
