@@ -1,0 +1,171 @@
+"""Benchmark of the fused MoE-layer forward on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu-baseline]
+
+A step is one forward of the layer (one persistent kernel launch) over one batch of synthetic
+tokens already resident in HBM. Prints one JSON line: latency per forward, the roofline of the
+launch (algorithmic FLOPs / event-timed duration vs dense bf16 MFMA peak), per-phase figures from
+the phased mode, and the CPU oracle timed on this box's host cores as a baseline.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0     # MI355X dense bf16 MFMA
+PEAK_FP32_TFLOPS = 157.3
+PEAK_HBM_GBS = 8000.0
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=32)
+    ap.add_argument("--warmup", type=int, default=32)
+    ap.add_argument("--workload", default="headline_e64_zipf")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--seed", type=int, default=0)
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures the single-GPU path (expert-parallel degree 1) only; run it with --gpus 1",
+              file=sys.stderr)
+        return 2
+
+    import numpy as np
+    import torch
+
+    import aristos_amd as ka
+    from aristos_amd import synth
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        return 2
+    torch.cuda.set_device(0)
+    w = synth.WORKLOADS[args.workload]
+    iP, d = synth.make_inputs(w, seed=args.seed, device="cuda")
+    torch.cuda.synchronize()
+    bf16 = d.elem_bytes == 2
+
+    ka.initialize(w.config)
+    try:
+        oP = synth.alloc_outputs(d)
+        # ---- fused mode: the product path
+        ka.moe.set_mode(ka.MODE_FUSED)
+        for _ in range(args.warmup):
+            ka.moe.forward_host(iP, oP)
+        ka.moe.stream_synchronize()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            ka.moe.forward_host(iP, oP)
+        ka.moe.stream_synchronize()
+        torch.cuda.synchronize()
+        wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+        # the same launches, timed by HIP events on the library stream (reference protocol, moe.cuh:160-181)
+        ev_ms = ka.moe.forward_host_bench(iP, oP, skip=0, trials=args.steps)
+        views = ka.moe.debug_views(d)
+        kept = int(np.minimum(views["expert_count"].astype(np.int64), d.kept_capacity).sum())
+        dropped = int((views["topk_slot"] < 0).sum())
+        hottest = float(views["expert_count"].max() / (d.S * d.k / d.E))
+        # ---- phased mode: the same device code, one launch per phase, for per-phase figures
+        ka.moe.set_mode(ka.MODE_PHASED)
+        ph_total = ka.moe.forward_host_bench(iP, oP, skip=max(2, args.warmup // 4), trials=max(4, args.steps))
+        ph = ka.moe.phase_times()
+        ka.moe.set_mode(ka.MODE_FUSED)
+    finally:
+        ka.finalize()
+
+    flops_layer = synth.layer_flops(d, kept)
+    flops_expert = synth.expert_flops(d, kept)
+    eb = d.elem_bytes
+    peak = PEAK_BF16_TFLOPS if bf16 else PEAK_FP32_TFLOPS
+    achieved = flops_layer / (ev_ms * 1e-3) / 1e12
+    up_dn_ms = ph["up"] + ph["down"]
+    phases = {
+        "total_ms": round(ph_total, 4),
+        "gate_ms": round(ph["gate"], 4), "slots_ms": round(ph["slots"], 4), "up_ms": round(ph["up"], 4),
+        "down_ms": round(ph["down"], 4), "combine_ms": round(ph["combine"], 4),
+        "expert_gemm_tflops": round(flops_expert / (up_dn_ms * 1e-3) / 1e12, 2) if up_dn_ms > 0 else None,
+        "expert_gemm_mfma_frac": round(flops_expert / (up_dn_ms * 1e-3) / 1e12 / peak, 4) if up_dn_ms > 0 else None,
+        # gate streams x once; combine reads T rows and writes S rows
+        "gate_hbm_gbs": round((d.S * d.H * eb + d.E * d.H * eb) / (ph["gate"] * 1e-3) / 1e9, 1) if ph["gate"] > 0 else None,
+        "combine_hbm_gbs": round((kept * d.H * eb + d.S * d.H * eb) / (ph["combine"] * 1e-3) / 1e9, 1) if ph["combine"] > 0 else None,
+    }
+
+    cpu = None
+    if not args.no_cpu_baseline:
+        cpu = cpu_baseline(w, iP, d, kept)
+
+    line = {
+        "metric": "moe_layer_fwd_latency_us",
+        "value": round(wall_ms * 1e3, 2),
+        "unit": "us",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(wall_ms, 5),
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16" if bf16 else "f32",
+        "data": "synthetic",
+        "config": {"workload": f"{w.name}: {w.note}", "S": d.S, "H": d.H, "I": d.I, "E": d.E, "top_k": d.k,
+                   "capacity_factor": w.config.capacity_factor, "EC": d.EC, "kept_pairs": kept,
+                   "dropped_pairs": dropped, "hottest_expert_vs_mean": round(hottest, 2),
+                   "mode": "fused persistent kernel, 1 launch per forward"},
+        "tokens_per_s": round(d.S / (wall_ms * 1e-3), 1),
+        "event_ms_per_step": round(ev_ms, 5),
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
+                     "frac": round(achieved / peak, 4), "traffic": None,
+                     "kernel": "fused_kernel (whole layer: gate + slots + expert GEMMs + combine)",
+                     "flops_per_launch": flops_layer},
+        "phases": phases,
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(line))
+    return 0
+
+
+def cpu_baseline(w, iP, d, kept):
+    """The CPU oracle (a port of the reference semantics, OpenMP) on this box's host cores. The
+    sample is a prefix of the tokens sized to a few seconds of CPU work; its time is scaled to the
+    whole layer by kept (token, expert) pairs, the gate being evaluated in full."""
+    import numpy as np
+    import torch
+    from oracle import moe_ref
+
+    c = moe_ref.cfg_from_keys(w.config)
+    if d.elem_bytes == 2:
+        iP_np = iP.view(torch.int16).cpu().numpy().view(np.uint16)
+    else:
+        iP_np = iP.cpu().numpy()
+    # routing pass (cheap) to pick the sample: a prefix of the tokens worth ~150 GFLOP of expert work
+    t0 = time.perf_counter()
+    route = moe_ref.forward(c, iP_np, token_mask=np.zeros(c.S, np.uint8))
+    gate_s = time.perf_counter() - t0
+    target_pairs = max(64, min(kept, int(150e9 / (4.0 * d.H * d.I))))
+    frac = min(1.0, target_pairs / max(kept, 1))
+    mask = np.zeros(c.S, np.uint8)
+    n_tok = max(1, int(round(c.S * frac)))
+    mask[:n_tok] = 1
+    sampled_pairs = int(((route["topk_slot"] >= 0) & (mask[:, None] == 1)).sum())
+    t0 = time.perf_counter()
+    moe_ref.forward(c, iP_np, logits=route["logits"], token_mask=mask)
+    ffn_s = time.perf_counter() - t0
+    scale = kept / max(sampled_pairs, 1)
+    total_s = gate_s + ffn_s * scale
+    return {"value": round(total_s * 1e6, 1), "unit": "us", "cores": moe_ref.threads(), "kind": "port",
+            "sample": f"gate+routing on all {c.S} tokens ({gate_s:.2f} s) + expert FFN and combine on "
+                      f"the first {int(mask.sum())} tokens = {sampled_pairs} of {kept} kept (token, expert) pairs "
+                      f"({ffn_s:.2f} s), scaled by {scale:.2f}",
+            "gflops": round((2.0 * d.S * d.H * d.E + 4.0 * kept * d.H * d.I) / total_s / 1e9, 1)}
+
+
+if __name__ == "__main__":
+    sys.exit(main())
