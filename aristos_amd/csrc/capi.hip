@@ -71,6 +71,19 @@ ArenaLayout layout_arena(const kleos_config_t& c, uint32_t n_tiles, uint32_t n_s
     return L;
 }
 
+// After a synchronisation: did a persistent kernel give up waiting on its scheduler counters?
+int check_scheduler(Context& c) {
+    uint32_t flag = 0;
+    hipError_t e = hipMemcpy(&flag, c.base.sched + sched_error_word(), 4, hipMemcpyDeviceToHost);
+    if (e != hipSuccess) return fail(KLEOS_EHIP, "scheduler check: %s", hipGetErrorString(e));
+    if (flag) {
+        (void)hipMemset(c.base.sched + sched_error_word(), 0, 4);
+        return fail(KLEOS_EHIP, "persistent kernel: a bounded wait on the tile scheduler expired; "
+                                "the outputs of that launch are invalid");
+    }
+    return KLEOS_OK;
+}
+
 int require_ctx(const char* who) {
     if (!g_ctx) return fail(KLEOS_ESTATE, "%s: Not initialized!", who);
     return KLEOS_OK;
@@ -284,13 +297,14 @@ extern "C" int kleos_moe_forward_bench(const void* iP, void* oP, uint32_t skip, 
     (void)hipEventDestroy(start);
     (void)hipEventDestroy(stop);
     for (auto& e : ev) (void)hipEventDestroy(e);
+    if (rc == KLEOS_OK) rc = check_scheduler(c);
     return rc;
 }
 
 extern "C" int kleos_stream_synchronize(void) {
     if (int rc = require_ctx("kleos_stream_synchronize")) return rc;
     KLEOS_HIP(hipStreamSynchronize(g_ctx->stream));
-    return KLEOS_OK;
+    return check_scheduler(*g_ctx);
 }
 
 extern "C" void* kleos_stream(void) { return g_ctx ? static_cast<void*>(g_ctx->stream) : nullptr; }

@@ -138,7 +138,11 @@ __global__ __launch_bounds__(kThreads) void combine_kernel(const LayerParams p) 
 //   [0..2]                 grid-barrier arrival counters, monotonically increasing across launches
 //   [8..15]                ticket counter of each XCD queue
 //   [16 .. 16+E*mt_max)    readiness: up-projection tiles stored per (expert, row block)
-constexpr uint32_t kSchedBar = 0, kSchedTicket = 8, kSchedReady = 16;
+//   [4]                    set to non-zero by a workgroup whose bounded wait expired
+constexpr uint32_t kSchedBar = 0, kSchedError = 4, kSchedTicket = 8, kSchedReady = 16;
+// Every wait in the persistent kernel is bounded so that the grid always drains: after this many
+// ticks of the 100 MHz wall clock a waiter records an error and proceeds.
+constexpr unsigned long long kWaitTicks = 300000000ull;   // 3 s
 // LDS header of the expert phase (bytes)
 constexpr size_t kLdsMt = 512, kLdsQueue = 128, kLdsSeg = 8 * (2 * 16 * kMaxGateGroups);
 constexpr size_t kFusedLdsHeader = kLdsMt + kLdsQueue + kLdsSeg;
@@ -150,12 +154,27 @@ struct Segment {
     uint32_t start;     // first ticket of the segment inside its queue
 };
 
-__device__ __forceinline__ void grid_barrier(uint32_t* ctr, uint32_t target) {
+// Spins (thread 0 only) until pred() holds or the wait bound expires.
+template <typename Pred>
+__device__ __forceinline__ void bounded_wait(uint32_t* sched, Pred&& pred) {
+    if (pred()) return;
+    const unsigned long long t0 = wall_clock64();
+    while (!pred()) {
+        __builtin_amdgcn_s_sleep(2);
+        if (wall_clock64() - t0 > kWaitTicks) {
+            atomic_store_relaxed(sched + kSchedError, 1u);
+            return;
+        }
+    }
+}
+
+__device__ __forceinline__ void grid_barrier(uint32_t* sched, uint32_t which, uint32_t target) {
+    uint32_t* ctr = sched + kSchedBar + which;
     __syncthreads();
     if (threadIdx.x == 0) {
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
         atomic_add_agent(ctr, 1u);
-        while (int32_t(atomic_load_relaxed(ctr) - target) < 0) __builtin_amdgcn_s_sleep(2);
+        bounded_wait(sched, [&] { return int32_t(atomic_load_relaxed(ctr) - target) >= 0; });
     }
     __syncthreads();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
@@ -178,7 +197,7 @@ __global__ __launch_bounds__(kThreads) void fused_kernel(const LayerParams p, ui
     }
     for (uint32_t tile = blockIdx.x; tile < p.n_gate_tiles; tile += nwg)
         gate_tile<T, NG>(p, tile, reinterpret_cast<float*>(smem));
-    grid_barrier(sched + kSchedBar + 0, barrier_base + nwg);
+    grid_barrier(sched, 0, barrier_base + nwg);
 
     // ---- phase 1: slots in token order
     {
@@ -188,7 +207,7 @@ __global__ __launch_bounds__(kThreads) void fused_kernel(const LayerParams p, ui
         uint32_t* other = p.super_count + size_t((p.epoch & 1u) ^ 1u) * p.n_super * p.E;
         for (uint32_t i = blockIdx.x * kThreads + tid; i < p.n_super * p.E; i += nwg * kThreads) other[i] = 0u;
     }
-    grid_barrier(sched + kSchedBar + 1, barrier_base + nwg);
+    grid_barrier(sched, 1, barrier_base + nwg);
 
     // ---- phase 2: expert tiles from per-XCD ticket queues
     // LDS map: row blocks per expert | queue starts, totals, task | segments | GEMM tile
@@ -252,7 +271,7 @@ __global__ __launch_bounds__(kThreads) void fused_kernel(const LayerParams p, ui
             if (kind == 1) {
                 // wait until every up-projection tile of this row block is stored
                 const uint32_t* ready = sched + kSchedReady + e * mt_max + mtile;
-                while (atomic_load_relaxed(ready) < tn_up) __builtin_amdgcn_s_sleep(4);
+                bounded_wait(sched, [&] { return atomic_load_relaxed(ready) >= tn_up; });
             }
             s_task[0] = e; s_task[1] = kind; s_task[2] = mtile; s_task[3] = ntile;
         }
@@ -267,7 +286,7 @@ __global__ __launch_bounds__(kThreads) void fused_kernel(const LayerParams p, ui
             atomic_add_agent(sched + kSchedReady + e * mt_max + mtile, 1u);
         }
     }
-    grid_barrier(sched + kSchedBar + 2, barrier_base + nwg);
+    grid_barrier(sched, 2, barrier_base + nwg);
 
     // ---- phase 3: combine, one token per wavefront
     for (uint32_t token = blockIdx.x * 4 + wave; token < p.S; token += nwg * 4) combine_token<T>(p, token);
@@ -310,6 +329,8 @@ const char* unsupported_reason(uint32_t E, uint32_t k) {
     if (E > 16 * kMaxGateGroups) return "num_experts > 256 is not supported by the gate kernel of this build";
     return nullptr;
 }
+
+uint32_t sched_error_word() { return kSchedError; }
 
 size_t sched_words(uint32_t E, uint32_t cap_rows) {
     return kSchedReady + size_t(E) * ceil_div_u32(cap_rows, 64) + 64;

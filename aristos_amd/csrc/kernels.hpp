@@ -8,6 +8,8 @@ namespace kleos_amd {
 
 // Number of uint32 scheduler words the persistent kernel needs for a layer with these sizes.
 size_t sched_words(uint32_t E, uint32_t cap_rows);
+// Index of the word a persistent kernel sets when one of its bounded waits expired.
+uint32_t sched_error_word();
 
 // Phase launchers (KLEOS_MODE_PHASED). dtype: 0 fp32, 2 bf16.
 hipError_t launch_gate(const LayerParams& p, int dtype, hipStream_t s);

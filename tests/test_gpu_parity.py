@@ -90,6 +90,7 @@ def check_against_oracle(c, keys, iP_np, mode, launches=1, token_mask=None, logi
 
 
 MODES = [ka.MODE_PHASED, ka.MODE_FUSED]
+MODE_IDS = ["phased", "fused"]
 
 
 def _keys(S, H, I, E, k, cf=1.0, drop=1, act=0, dt=2):
@@ -98,7 +99,7 @@ def _keys(S, H, I, E, k, cf=1.0, drop=1, act=0, dt=2):
 
 
 # ------------------------------------------------------------------ the reference's CPU-sized case
-@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("mode", MODES, ids=MODE_IDS)
 def test_tiny_fp32_config(mode):
     """S=128 H=256 I=512 E=8 top-2 cf=1.0 fp32, seed 0."""
     w = synth.WORKLOADS["tiny_fp32"]
@@ -134,7 +135,7 @@ CASES = [
 ]
 
 
-@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("mode", MODES, ids=MODE_IDS)
 @pytest.mark.parametrize("S,H,I,E,k,cf,drop,act,dt,bias", CASES)
 def test_shapes_and_edges(mode, S, H, I, E, k, cf, drop, act, dt, bias):
     keys = _keys(S, H, I, E, k, cf, drop, act, dt)
@@ -148,7 +149,7 @@ def test_shapes_and_edges(mode, S, H, I, E, k, cf, drop, act, dt, bias):
     check_against_oracle(c, keys, iP, mode)
 
 
-@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("mode", MODES, ids=MODE_IDS)
 def test_exact_ties_go_to_the_lower_index(mode):
     """Duplicate gate rows give bit-identical logits for expert pairs; the lower index must win, and
     an all-equal row must select experts 0..k-1."""
@@ -170,7 +171,7 @@ def test_exact_ties_go_to_the_lower_index(mode):
         if 11 in sel: assert 7 in sel and sel.index(7) < sel.index(11)
 
 
-@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("mode", MODES, ids=MODE_IDS)
 def test_everything_routed_to_two_experts(mode):
     """Heavy overflow: every token prefers experts 0 and 1, the rest of the batch is dropped whole."""
     keys = _keys(512, 128, 128, 8, 2, dt=0)
@@ -184,7 +185,7 @@ def test_everything_routed_to_two_experts(mode):
     assert (moe_out[128:] == 0).all()
 
 
-@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("mode", MODES, ids=MODE_IDS)
 def test_identity_experts_return_input(mode):
     """The reference author's own check (csrc/main.cu:16): identity expert weights."""
     keys = _keys(256, 128, 128, 8, 2, cf=8.0, dt=0)
@@ -198,7 +199,7 @@ def test_identity_experts_return_input(mode):
 
 
 # ------------------------------------------------------------------ back-to-back launches
-@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("mode", MODES, ids=MODE_IDS)
 def test_back_to_back_launches_need_no_host_reset(mode):
     """The reference resets its state inside the kernel (moe.cuh:31-70) so launches can follow each
     other; here the same must hold for counters and the double-buffered histograms. Five launches,
@@ -242,7 +243,7 @@ def _full_size(name, mode, n_check, seed=0):
     return c, w, iP_np, mask
 
 
-@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("mode", MODES, ids=MODE_IDS)
 def test_balanced_e16_full_size(mode):
     """S=4096 H=I=2048 E=16 top-2 bf16, balanced load."""
     c, w, iP_np, mask = _full_size("balanced_e16", mode, 256)
@@ -251,7 +252,7 @@ def test_balanced_e16_full_size(mode):
     assert counts.sum() == c.S * c.k and counts.max() < 1.3 * counts.mean()
 
 
-@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("mode", MODES, ids=MODE_IDS)
 def test_headline_e64_zipf_full_size(mode):
     """S=8192 H=I=2048 E=64 top-2 bf16 with the Zipf logit bias: the hottest expert is routed about
     four times the mean load, so tokens are dropped and the scheduler sees unequal experts."""
