@@ -5,6 +5,8 @@
 // (csrc/include/kleos/moe/moe.cuh:146-205), for one GPU and expert-parallel degree 1.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
+#include <cstdlib>
 #include <cstring>
 #include <vector>
 
@@ -39,11 +41,13 @@ Context* g_ctx = nullptr;   // one context per process, like the reference's glo
                         hipGetErrorName(e_), hipGetErrorString(e_));                            \
     } while (0)
 
+constexpr uint32_t kMaxWorkgroups = 1024;   // persistent grid never exceeds CUs x 2
+
 size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 struct ArenaLayout {
     size_t logits, topk_expert, topk_prob, combine_den, topk_slot, tile_count, super_count,
-        expert_count, slot_token, h1, y, sched, total;
+        expert_count, slot_token, h1, y, sched, stamps, total;
     size_t zero_begin, zero_end;   // range that must start as zeros
 };
 
@@ -57,6 +61,7 @@ ArenaLayout layout_arena(const kleos_config_t& c, uint32_t n_tiles, uint32_t n_s
     L.super_count = take(2 * size_t(n_super) * E * 4);
     L.sched = take(sched_words(c.E, c.cap_rows) * 4);
     L.expert_count = take(E * 4);
+    L.stamps = take(size_t(kMaxWorkgroups) * 8 * 8);
     L.zero_end = off;
     L.logits = take(S * E * 4);
     L.topk_expert = take(S * k * 4);
@@ -193,7 +198,9 @@ extern "C" int kleos_initialize_cfg(const kleos_config_t* user_cfg) {
     p.h1 = a + L.h1;
     p.y = a + L.y;
     p.sched = reinterpret_cast<uint32_t*>(a + L.sched);
+    p.stamps = reinterpret_cast<unsigned long long*>(a + L.stamps);
     KLEOS_HIP_BAIL(plan_fused(p, int(cfg.torch_dtype), c->num_cus, &c->plan));
+    if (c->plan.nwg > kMaxWorkgroups) return bail(fail(KLEOS_EUNSUPPORTED, "persistent grid of %u workgroups exceeds %u", c->plan.nwg, kMaxWorkgroups));
 #undef KLEOS_HIP_BAIL
     g_ctx = c;
     return KLEOS_OK;
@@ -283,6 +290,22 @@ extern "C" int kleos_moe_forward_bench(const void* iP, void* oP, uint32_t skip, 
         KLEOS_HIP(hipEventElapsedTime(&ms, start, stop));
         *ms_per_launch = ms / float(trials);                          // moe.cuh:181
         for (float& v : c.phase_ms) v = 0.f;
+        if (!phased) {
+            // phase boundaries of the last launch, stamped by every workgroup of the persistent kernel
+            std::vector<unsigned long long> st(size_t(c.plan.nwg) * 8);
+            KLEOS_HIP(hipMemcpy(st.data(), c.base.stamps, st.size() * 8, hipMemcpyDeviceToHost));
+            unsigned long long t0 = ~0ull, b[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+            for (uint32_t w = 0; w < c.plan.nwg; ++w) {
+                t0 = std::min(t0, st[size_t(w) * 8]);
+                for (int i = 0; i < 8; ++i) b[i] = std::max(b[i], st[size_t(w) * 8 + i]);
+            }
+            const float tick_ms = 1e-5f;   // 100 MHz
+            c.phase_ms[0] = float(b[2] - t0) * tick_ms;        // gate, through the first grid barrier
+            c.phase_ms[1] = float(b[4] - b[2]) * tick_ms;      // slots, through the second
+            c.phase_ms[2] = float(b[6] - b[4]) * tick_ms;      // both projections, through the third
+            c.phase_ms[3] = 0.f;
+            c.phase_ms[4] = float(b[7] - b[6]) * tick_ms;      // combine
+        }
         if (phased) {
             for (uint32_t i = 0; i < trials; ++i)
                 for (int ph = 0; ph < 5; ++ph) {

@@ -12,59 +12,110 @@
 namespace kleos_amd {
 
 // ------------------------------------------------------------------------------------------------
-// bf16, matrix cores. 256 threads = 4 wavefronts arranged WAVES_M x WAVES_N over a BM x BN tile;
-// K is walked in slices of 64 through a double-buffered, XOR-swizzled LDS tile (rows of 128 bytes,
-// 16-byte chunk c of row r stored at chunk position c ^ (r & 7), which makes both the 16-byte
-// stores of the staging pass and the ds_read_b128 fragment loads bank-conflict free).
+// bf16, matrix cores. WAVES_M x WAVES_N wavefronts over a BM x BN tile (two wavefronts per SIMD with
+// eight of them, so that one's LDS waits hide behind the other's matrix instructions).
+//
+// K is walked in slices of 64 through a ring of LDS stages that the wavefronts fill with direct
+// global->LDS loads (global_load_lds_dwordx4: each lane names a 16-byte global source, the 64 lanes
+// of the instruction land in 1 KB of consecutive LDS). The loads of the next slice are issued
+// before the current slice is multiplied, so they have a whole slice of matrix work to arrive and
+// never occupy a vector register. A slice holds 128 bytes of every row, i.e. whole cache lines:
+// narrower slices make consecutive loads hit lines whose miss is still pending, which stalls the
+// L1. Rows of A are gathered through the slot->token table by giving each lane its token's row
+// address.
+//
+// LDS layout of a stage: rows of 128 bytes (64 bf16), 16-byte chunk c of row r stored at chunk
+// position c ^ swz(r). The LDS of gfx950 has 64 banks of 4 bytes (two tile rows per bank row) and
+// serves a 16-byte access of 16 lanes per clock; with this swizzle any 16 consecutive rows read at
+// one chunk index cover all 64 banks. Because the LDS destination of a direct load is fixed by the
+// lane number, the swizzle is applied on the global side: lane (r, p) fetches chunk p ^ swz(r) of
+// its row.
 //
 // The weight rows feed the matrix core's row operand and the activation rows its column operand,
-// i.e. the core computes C^T: a lane then owns 4 consecutive output columns of one output row and
-// the epilogue packs them into one 8-byte store.
+// i.e. the core computes C^T: a lane then owns 4 consecutive output columns of one output row.
 // ------------------------------------------------------------------------------------------------
 constexpr int kGemmBK = 64;
+constexpr int kGemmStages = 2;
+#ifdef KLEOS_TRACE
+__device__ unsigned long long* g_trace = nullptr;   // diagnostic build only
+#endif
+
+__device__ __forceinline__ int swz(int r) { return ((r >> 1) & 7) ^ ((r & 1) << 2); }
 
 template <int BM, int BN>
-constexpr int gemm_bf16_smem_bytes() { return 2 * (BM + BN) * kGemmBK * 2; }
+constexpr int gemm_bf16_smem_bytes() { return kGemmStages * (BM + BN) * kGemmBK * 2; }
 
-template <int ACT, int BM, int BN, int WAVES_M, int WAVES_N>
+typedef const __attribute__((address_space(1))) void* global_cptr;
+typedef __attribute__((address_space(3))) void* lds_ptr;
+
+// Waits until at most N of this wavefront's vector-memory operations are outstanding.
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+    static_assert(N >= 0 && N < 64);
+    // s_waitcnt simm16: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] at [15:14]
+    __builtin_amdgcn_s_waitcnt(0x0f70 | (N & 15) | ((N >> 4) << 14));
+}
+
+// A_AUX: cache-policy bits of the loads of A (0 = default, 1 = sc0: do not trust this CU's L1, for
+// rows another workgroup of the same launch has just written).
+template <int ACT, int BM, int BN, int WAVES_M, int WAVES_N, int A_AUX>
 __device__ __forceinline__ void gemm_tile_bf16(
     const bf16_t* __restrict__ a_base, const int32_t* __restrict__ a_row_index, uint32_t lda,
     uint32_t m_valid,
     const bf16_t* __restrict__ b_base, uint32_t ldb, uint32_t n_valid,
     const bf16_t* __restrict__ bias, bf16_t* __restrict__ c_base, uint32_t ldc, uint32_t K,
     char* smem) {
-    static_assert(WAVES_M * WAVES_N == 4, "four wavefronts per workgroup");
+    constexpr int kGemmWaves = WAVES_M * WAVES_N;
     constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;   // wavefront tile
     constexpr int TM = WM / 32, TN = WN / 32;             // 32x32 matrix-core tiles per wavefront
-    static_assert(WM % 32 == 0 && WN % 32 == 0 && BM % 32 == 0 && BN % 32 == 0);
-    constexpr int PA = BM / 32, PB = BN / 32;             // staging passes (32 rows x 8 chunks each)
-    constexpr int kABytes = BM * kGemmBK * 2, kBBytes = BN * kGemmBK * 2;
+    static_assert(WM % 32 == 0 && WN % 32 == 0);
+    constexpr int kRowBytes = kGemmBK * 2;                // 128
+    constexpr int kABytes = BM * kRowBytes, kBBytes = BN * kRowBytes;
     constexpr int kStage = kABytes + kBBytes;
+    // one direct load covers 8 rows (1 KB); each wavefront issues LA + LB of them per stage
+    static_assert(BM % (8 * kGemmWaves) == 0 && BN % (8 * kGemmWaves) == 0);
+    constexpr int LA = BM / (8 * kGemmWaves), LB = BN / (8 * kGemmWaves);
+    constexpr int kLoadsPerStage = LA + LB;
 
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
     const int wm = wave / WAVES_N, wn = wave % WAVES_N;
-    const int ld_row = tid >> 3, ld_ch = tid & 7;
 
-    // Source row pointers of this thread's staging chunks; nullptr rows are staged as zeros.
-    const bf16_t* pa[PA];
-    const bf16_t* pb[PB];
+    // Global source of this lane for each of its direct loads. Rows past the valid range re-read
+    // the last valid row: their products land in accumulator rows / columns that are never stored.
+    const int ld_r = lane >> 3, ld_p = lane & 7;
+    const bf16_t* pa[LA];
+    const bf16_t* pb[LB];
 #pragma unroll
-    for (int i = 0; i < PA; ++i) {
-        const uint32_t r = ld_row + 32 * i;
-        if (r < m_valid) {
-            const size_t src = a_row_index ? size_t(a_row_index[r]) : size_t(r);
-            pa[i] = a_base + src * lda + ld_ch * 8;
-        } else {
-            pa[i] = nullptr;
-        }
+    for (int i = 0; i < LA; ++i) {
+        const int row = 8 * (wave + kGemmWaves * i) + ld_r;
+        uint32_t r = row < int(m_valid) ? row : m_valid - 1;
+        const size_t src = a_row_index ? size_t(a_row_index[r]) : size_t(r);
+        pa[i] = a_base + src * lda + ((ld_p ^ swz(row)) << 3);
     }
 #pragma unroll
-    for (int i = 0; i < PB; ++i) {
-        const uint32_t r = ld_row + 32 * i;
-        pb[i] = r < n_valid ? b_base + size_t(r) * ldb + ld_ch * 8 : nullptr;
+    for (int i = 0; i < LB; ++i) {
+        const int row = 8 * (wave + kGemmWaves * i) + ld_r;
+        uint32_t r = row < int(n_valid) ? row : n_valid - 1;
+        pb[i] = b_base + size_t(r) * ldb + ((ld_p ^ swz(row)) << 3);
     }
-    const int st_off = ld_row * 128 + ((ld_ch ^ (ld_row & 7)) << 4);   // + 32*i rows = + 4096*i bytes
+    // part `part` of `parts` of the direct loads that bring slice kt into `stage`
+    auto issue_part = [&](uint32_t kt, int stage, int part, int parts) {
+        char* sa = smem + stage * kStage;
+        char* sb = sa + kABytes;
+        const uint32_t k0 = kt * kGemmBK;
+#pragma unroll
+        for (int i = 0; i < LA; ++i)
+            if (i * parts / LA == part)
+                __builtin_amdgcn_global_load_lds((global_cptr)(pa[i] + k0),
+                                                 (lds_ptr)(sa + 1024 * (wave + kGemmWaves * i)), 16, 0, A_AUX);
+#pragma unroll
+        for (int i = 0; i < LB; ++i)
+            if (i * parts / LB == part)
+                __builtin_amdgcn_global_load_lds((global_cptr)(pb[i] + k0),
+                                                 (lds_ptr)(sb + 1024 * (wave + kGemmWaves * i)), 16, 0, 0);
+    };
+    auto issue = [&](uint32_t kt, int stage) { issue_part(kt, stage, 0, 1); };
 
     f32x16 acc[TN][TM];
 #pragma unroll
@@ -74,80 +125,127 @@ __device__ __forceinline__ void gemm_tile_bf16(
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[ni][mi][v] = 0.f;
 
-    u32x4 ra[PA], rb[PB];
-    auto fetch = [&](uint32_t k0) {
-#pragma unroll
-        for (int i = 0; i < PA; ++i) ra[i] = pa[i] ? load16(pa[i] + k0) : u32x4{0u, 0u, 0u, 0u};
-#pragma unroll
-        for (int i = 0; i < PB; ++i) rb[i] = pb[i] ? load16(pb[i] + k0) : u32x4{0u, 0u, 0u, 0u};
-    };
-    auto stage = [&](int buf) {
-        char* sa = smem + buf * kStage;
-        char* sb = sa + kABytes;
-#pragma unroll
-        for (int i = 0; i < PA; ++i) store16(sa + st_off + i * 4096, ra[i]);
-#pragma unroll
-        for (int i = 0; i < PB; ++i) store16(sb + st_off + i * 4096, rb[i]);
-    };
-
     const uint32_t k_tiles = K / kGemmBK;
-    fetch(0);
-    stage(0);
-    __syncthreads();
+    // prologue: the first kGemmStages - 1 slices in flight
+#pragma unroll
+    for (int st = 0; st < kGemmStages - 1; ++st)
+        if (uint32_t(st) < k_tiles) issue(st, st);
 
     const int fr_row = lane & 31, fr_half = lane >> 5;
-    for (uint32_t kt = 0; kt < k_tiles; ++kt) {
-        const int buf = kt & 1;
-        if (kt + 1 < k_tiles) fetch((kt + 1) * kGemmBK);
-        const char* sa = smem + buf * kStage;
-        const char* sb = sa + kABytes;
+    constexpr int kSteps = kGemmBK / 16;   // matrix instructions consume 16 values of K
+    // fragment byte offsets inside a stage for every K step of a slice
+    int off_w[TN][kSteps], off_x[TM][kSteps];
 #pragma unroll
-        for (int ks = 0; ks < kGemmBK / 16; ++ks) {
-            const int ch = ks * 2 + fr_half;
+    for (int ni = 0; ni < TN; ++ni) {
+        const int r = wn * WN + ni * 32 + fr_row;
+#pragma unroll
+        for (int ks = 0; ks < kSteps; ++ks) off_w[ni][ks] = kABytes + r * kRowBytes + (((ks * 2 + fr_half) ^ swz(r)) << 4);
+    }
+#pragma unroll
+    for (int mi = 0; mi < TM; ++mi) {
+        const int r = wm * WM + mi * 32 + fr_row;
+#pragma unroll
+        for (int ks = 0; ks < kSteps; ++ks) off_x[mi][ks] = r * kRowBytes + (((ks * 2 + fr_half) ^ swz(r)) << 4);
+    }
+
+#ifdef KLEOS_TRACE
+    unsigned long long* trc = (blockIdx.x == KLEOS_TRACE && lane == 0 && g_trace) ? g_trace + wave * 256 : nullptr;
+#define KTR(i) if (trc && kt < 32) trc[kt * 6 + (i)] = __builtin_readcyclecounter()
+#else
+#define KTR(i)
+#endif
+    for (uint32_t kt = 0; kt < k_tiles; ++kt) {
+        KTR(0);
+        // This wavefront's loads of slice kt have landed once only those of the later slices in
+        // flight (kGemmStages - 2 of them, fewer at the end) are outstanding.
+        if constexpr (kGemmStages == 2) {
+            wait_vmcnt<0>();
+        } else {
+            static_assert(kGemmStages == 2 || kGemmStages == 3 || kGemmStages == 4);
+            const uint32_t later = k_tiles - 1 - kt;   // slices after kt that exist
+            if (later >= uint32_t(kGemmStages - 2)) wait_vmcnt<(kGemmStages - 2) * kLoadsPerStage>();
+            else if (kGemmStages == 4 && later == 1) wait_vmcnt<kLoadsPerStage>();
+            else wait_vmcnt<0>();
+        }
+        // every wavefront's share of slice kt is in LDS, and everyone has finished reading slice
+        // kt-1, whose stage the next loads overwrite
+        KTR(1);
+        asm volatile("s_barrier" ::: "memory");
+        KTR(2);
+        // The loads of the next slice are spread over the K steps of this one: issued in one
+        // burst they queue up in the texture addresser and hold the wavefront (and with it its
+        // matrix instructions) until the last one is accepted.
+        const bool more = kt + kGemmStages - 1 < k_tiles;
+        const uint32_t next_kt = kt + kGemmStages - 1;
+        const int next_stage = next_kt % kGemmStages;
+        KTR(3);
+        const char* st = smem + (kt % kGemmStages) * kStage;
+#pragma unroll
+        for (int ks = 0; ks < kSteps; ++ks) {
             bf16x8 fw[TN], fx[TM];
 #pragma unroll
-            for (int ni = 0; ni < TN; ++ni) {
-                const int r = wn * WN + ni * 32 + fr_row;
-                fw[ni] = __builtin_bit_cast(bf16x8, load16(sb + r * 128 + ((ch ^ (r & 7)) << 4)));
-            }
+            for (int ni = 0; ni < TN; ++ni) fw[ni] = __builtin_bit_cast(bf16x8, load16(st + off_w[ni][ks]));
 #pragma unroll
-            for (int mi = 0; mi < TM; ++mi) {
-                const int r = wm * WM + mi * 32 + fr_row;
-                fx[mi] = __builtin_bit_cast(bf16x8, load16(sa + r * 128 + ((ch ^ (r & 7)) << 4)));
-            }
+            for (int mi = 0; mi < TM; ++mi) fx[mi] = __builtin_bit_cast(bf16x8, load16(st + off_x[mi][ks]));
+            if (more) issue_part(next_kt, next_stage, ks, kSteps);
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int ni = 0; ni < TN; ++ni)
 #pragma unroll
                 for (int mi = 0; mi < TM; ++mi)
                     acc[ni][mi] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fw[ni], fx[mi], acc[ni][mi], 0, 0, 0);
         }
-        if (kt + 1 < k_tiles) stage(buf ^ 1);
-        __syncthreads();
+        KTR(4);
     }
+    // all wavefronts are done with the ring: each now reuses its own 1/8 of it
+    __syncthreads();
 
-    // Epilogue. acc[ni][mi][v]: output column n = wn*WN + ni*32 + 8*(v/4) + 4*(lane/32) + v%4,
-    // output row m = wm*WM + mi*32 + lane%32.
+    // Epilogue. acc[ni][mi][v] is output column n = wn*WN + ni*32 + 8*(v/4) + 4*(lane/32) + v%4 of
+    // output row m = wm*WM + mi*32 + lane%32: a lane owns 4 consecutive columns of 16 rows. Bias,
+    // activation and the rounding to Element happen in registers; the wavefront then transposes its
+    // WM x WN block through a private LDS region (rows of WN*2 bytes, 16-byte chunk c of row r at
+    // position c ^ ((r >> 1) & 7)) so that the global stores are 16 bytes per lane and cover whole
+    // 128-byte lines of the output rows.
+    static_assert(WN % 64 == 0, "epilogue staging works on 64-column (128-byte) panels");
+    static_assert(WM * WN * 2 * kGemmWaves <= gemm_bf16_smem_bytes<BM, BN>());
+    char* stg_wave = smem + wave * (WM * WN * 2);
 #pragma unroll
-    for (int ni = 0; ni < TN; ++ni) {
+    for (int pn = 0; pn < WN / 64; ++pn) {                  // 64-column panel of the wavefront tile
+        char* stg = stg_wave + pn * (WM * 128);
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const uint32_t n = wn * WN + ni * 32 + 8 * q + 4 * fr_half;
-            if (n >= n_valid) continue;
-            float bv[4];
-            const bf16x4 b4 = *reinterpret_cast<const bf16x4*>(bias + n);
+        for (int nl = 0; nl < 2; ++nl) {
+            const int ni = pn * 2 + nl;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) bv[j] = float(b4[j]);
+            for (int q = 0; q < 4; ++q) {
+                const uint32_t n = wn * WN + ni * 32 + 8 * q + 4 * fr_half;
+                float bv[4] = {0.f, 0.f, 0.f, 0.f};
+                if (n < n_valid) {
+                    const bf16x4 b4 = *reinterpret_cast<const bf16x4*>(bias + n);
 #pragma unroll
-            for (int mi = 0; mi < TM; ++mi) {
-                const uint32_t m = wm * WM + mi * 32 + fr_row;
-                if (m >= m_valid) continue;
-                bf16x4 o;
+                    for (int j = 0; j < 4; ++j) bv[j] = float(b4[j]);
+                }
 #pragma unroll
-                for (int j = 0; j < 4; ++j) o[j] = static_cast<bf16_t>(activate<ACT>(acc[ni][mi][4 * q + j] + bv[j]));
-                *reinterpret_cast<bf16x4*>(c_base + size_t(m) * ldc + n) = o;
+                for (int mi = 0; mi < TM; ++mi) {
+                    const int r = mi * 32 + fr_row;
+                    bf16x4 o;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) o[j] = static_cast<bf16_t>(activate<ACT>(acc[ni][mi][4 * q + j] + bv[j]));
+                    *reinterpret_cast<bf16x4*>(stg + r * 128 + (((nl * 4 + q) ^ ((r >> 1) & 7)) << 4) + fr_half * 8) = o;
+                }
             }
         }
+        // same wavefront wrote and reads the region: LDS operations of one wavefront complete in order
+#pragma unroll
+        for (int it = 0; it < WM * 8 / kWave; ++it) {
+            const int id = it * kWave + lane;
+            const int r = id >> 3, c = id & 7;
+            const u32x4 v = load16(stg + r * 128 + ((c ^ ((r >> 1) & 7)) << 4));
+            const uint32_t m = wm * WM + r, n = wn * WN + pn * 64 + c * 8;
+            if (m < m_valid && n < n_valid) store16(c_base + size_t(m) * ldc + n, v);
+        }
     }
+    // the caller may start the next tile's loads into the ring right away
+    __syncthreads();
 }
 
 // ------------------------------------------------------------------------------------------------

@@ -27,13 +27,15 @@ struct GateK {
 template <int NG>
 constexpr int gate_smem_floats() { return 3 * NG * 4 * kWave; }
 
-// One 16-token tile of the gate. Called by all 256 threads of a workgroup; the four waves split
-// the hidden dimension, wave 0 reduces the partial sums in a fixed order and runs the epilogue.
-// `smem` must hold gate_smem_floats<NG>() floats and may be reused after the call returns on all
-// threads followed by a workgroup barrier (the function ends with one).
+// One 16-token tile of the gate, computed by a group of four wavefronts (256 threads): the four
+// waves split the hidden dimension, wave 0 of the group reduces the partial sums in a fixed order
+// and runs the epilogue. A workgroup of 256*G threads runs G groups side by side on different
+// tiles; every thread of the workgroup must call the function (it contains workgroup barriers) and
+// a group without a tile passes valid = false. `smem` is the group's private scratch of
+// gate_smem_floats<NG>() floats; it may be reused after the call (which ends with a barrier).
 template <typename T, int NG>
-__device__ __forceinline__ void gate_tile(const LayerParams& p, uint32_t tile, float* smem) {
-    const int tid = threadIdx.x;
+__device__ __forceinline__ void gate_tile(const LayerParams& p, uint32_t tile, bool valid, float* smem) {
+    const int tid = threadIdx.x & 255;
     const int wave = tid >> 6, lane = tid & 63;
     const int col = lane & 15;       // token inside the tile / expert row inside a group
     const int chunk = lane >> 4;     // which 16-byte K chunk of a step this lane loads
@@ -53,7 +55,7 @@ __device__ __forceinline__ void gate_tile(const LayerParams& p, uint32_t tile, f
     for (int g = 0; g < NG; ++g) acc[g] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     // logits^T tile: experts are the matrix-core rows, tokens its columns (gate.cuh:526-534).
-    for (uint32_t s = s0; s < s1; ++s) {
+    for (uint32_t s = valid ? s0 : s1; s < s1; ++s) {
         const uint32_t off = s * kStepK;
         const u32x4 b = load16(xrow + off);
 #pragma unroll
@@ -63,7 +65,7 @@ __device__ __forceinline__ void gate_tile(const LayerParams& p, uint32_t tile, f
         }
     }
 
-    if (wave > 0) {
+    if (valid && wave > 0) {
         float* dst = smem + (wave - 1) * (NG * 4 * kWave);
 #pragma unroll
         for (int g = 0; g < NG; ++g)
@@ -71,7 +73,7 @@ __device__ __forceinline__ void gate_tile(const LayerParams& p, uint32_t tile, f
             for (int v = 0; v < 4; ++v) dst[(g * 4 + v) * kWave + lane] = acc[g][v];
     }
     __syncthreads();
-    if (wave == 0) {
+    if (valid && wave == 0) {
         // fixed summation order: wave 0 + wave 1 + wave 2 + wave 3
 #pragma unroll
         for (int w = 0; w < 3; ++w) {

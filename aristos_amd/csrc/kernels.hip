@@ -24,14 +24,18 @@ namespace kleos_amd {
 
 namespace {
 
-constexpr int kThreads = 256;
 constexpr int kXcds = 8;
 // expert GEMM tile of the bf16 path
-constexpr int kBM = 128, kBN = 128;
+constexpr int kBM = 256, kBN = 256;
+constexpr int kWavesM = 2, kWavesN = 4;   // wavefront grid over the tile
+constexpr int kGemmThreads = kWavesM * kWavesN * kWave;
 
+// Tile shape and workgroup size of the expert projections per Element type. The workgroup size is
+// also that of the persistent kernel, whose other phases run on groups of its wavefronts.
 template <typename T> struct TileShape;
-template <> struct TileShape<bf16_t> { static constexpr int BM = kBM, BN = kBN; };
-template <> struct TileShape<float> { static constexpr int BM = kF32Tile, BN = kF32Tile; };
+template <> struct TileShape<bf16_t> { static constexpr int BM = kBM, BN = kBN, kThreads = kGemmThreads; };
+template <> struct TileShape<float> { static constexpr int BM = kF32Tile, BN = kF32Tile, kThreads = 256; };
+constexpr int kPhaseThreads = 256;   // gate, slot and combine kernels of the phased mode
 
 template <typename T>
 constexpr int gemm_smem_bytes() {
@@ -69,7 +73,7 @@ __device__ __forceinline__ void expert_tile(const LayerParams& p, uint32_t e, ui
         auto run = [&](auto act_tag) {
             constexpr int ACT = decltype(act_tag)::value;
             if constexpr (sizeof(T) == 2)
-                gemm_tile_bf16<ACT, BM, BN, 2, 2>(a, idx, p.H, m_valid, w, K, n_valid, bias, c, p.I, K, smem);
+                gemm_tile_bf16<ACT, BM, BN, kWavesM, kWavesN, 0>(a, idx, p.H, m_valid, w, K, n_valid, bias, c, p.I, K, smem);
             else
                 gemm_tile_f32<ACT>(a, idx, p.H, m_valid, w, K, n_valid, bias, c, p.I, K, smem);
         };
@@ -79,7 +83,7 @@ __device__ __forceinline__ void expert_tile(const LayerParams& p, uint32_t e, ui
         const T* a = static_cast<const T*>(p.h1) + row_base * p.I;
         T* c = static_cast<T*>(p.y) + row_base * p.H + col0;
         if constexpr (sizeof(T) == 2)
-            gemm_tile_bf16<2, BM, BN, 2, 2>(a, nullptr, p.I, m_valid, w, K, n_valid, bias, c, p.H, K, smem);
+            gemm_tile_bf16<2, BM, BN, kWavesM, kWavesN, 1>(a, nullptr, p.I, m_valid, w, K, n_valid, bias, c, p.H, K, smem);
         else
             gemm_tile_f32<2>(a, nullptr, p.I, m_valid, w, K, n_valid, bias, c, p.H, K, smem);
     }
@@ -87,19 +91,19 @@ __device__ __forceinline__ void expert_tile(const LayerParams& p, uint32_t e, ui
 
 // ------------------------------------------------------------------------------------ phased
 template <typename T, int NG>
-__global__ __launch_bounds__(kThreads) void gate_kernel(const LayerParams p) {
+__global__ __launch_bounds__(kPhaseThreads) void gate_kernel(const LayerParams p) {
     __shared__ float smem[gate_smem_floats<NG>()];
-    gate_tile<T, NG>(p, blockIdx.x, smem);
+    gate_tile<T, NG>(p, blockIdx.x, true, smem);
 }
 
-__global__ __launch_bounds__(kThreads) void slot_kernel(const LayerParams p) {
+__global__ __launch_bounds__(kPhaseThreads) void slot_kernel(const LayerParams p) {
     extern __shared__ uint32_t slot_smem[];
     const uint32_t wave = threadIdx.x >> 6;
     const uint32_t tile = blockIdx.x * 4 + wave;
     slot_tile(p, tile, tile < p.n_gate_tiles, slot_smem + wave * p.E);
     // the coarse counts of the other epoch are free now: clear them for the next launch
     uint32_t* other = p.super_count + size_t((p.epoch & 1u) ^ 1u) * p.n_super * p.E;
-    for (uint32_t i = blockIdx.x * kThreads + threadIdx.x; i < p.n_super * p.E; i += gridDim.x * kThreads)
+    for (uint32_t i = blockIdx.x * kPhaseThreads + threadIdx.x; i < p.n_super * p.E; i += gridDim.x * kPhaseThreads)
         other[i] = 0u;
 }
 
@@ -108,7 +112,7 @@ __global__ __launch_bounds__(kThreads) void slot_kernel(const LayerParams p) {
 // rows meet in one L2. Row blocks vary fastest so that the tiles re-reading one weight tile run
 // together.
 template <typename T>
-__global__ __launch_bounds__(kThreads) void expert_gemm_kernel(const LayerParams p, uint32_t kind,
+__global__ __launch_bounds__(TileShape<T>::kThreads) void expert_gemm_kernel(const LayerParams p, uint32_t kind,
                                                                uint32_t tiles_m, uint32_t tiles_n) {
     extern __shared__ __attribute__((aligned(16))) char gemm_smem[];
     const uint32_t per_expert = tiles_m * tiles_n;
@@ -128,7 +132,7 @@ __global__ __launch_bounds__(kThreads) void expert_gemm_kernel(const LayerParams
 }
 
 template <typename T>
-__global__ __launch_bounds__(kThreads) void combine_kernel(const LayerParams p) {
+__global__ __launch_bounds__(kPhaseThreads) void combine_kernel(const LayerParams p) {
     const uint32_t token = blockIdx.x * 4 + (threadIdx.x >> 6);
     if (token < p.S) combine_token<T>(p, token);
 }
@@ -181,40 +185,49 @@ __device__ __forceinline__ void grid_barrier(uint32_t* sched, uint32_t which, ui
 }
 
 template <typename T, int NG>
-__global__ __launch_bounds__(kThreads) void fused_kernel(const LayerParams p, uint32_t barrier_base,
-                                                         uint32_t mt_max, uint32_t lag) {
+__global__ __launch_bounds__(TileShape<T>::kThreads) void fused_kernel(const LayerParams p, uint32_t barrier_base,
+                                                                      uint32_t mt_max, uint32_t lag) {
     static_assert(sizeof(Segment) == 8, "segment table sizing");
     extern __shared__ __attribute__((aligned(16))) char smem[];
     constexpr int BM = TileShape<T>::BM, BN = TileShape<T>::BN;
-    const uint32_t tid = threadIdx.x, wave = tid >> 6;
+    constexpr uint32_t kThreads = TileShape<T>::kThreads;
+    constexpr uint32_t kWaves = kThreads / kWave, kGroups = kThreads / 256;
+    const uint32_t tid = threadIdx.x, wave = tid >> 6, group = tid >> 8;
     const uint32_t nwg = gridDim.x;
     uint32_t* sched = p.sched;
+    unsigned long long* stamp = p.stamps + size_t(blockIdx.x) * 8;
+    if (tid == 0) stamp[0] = wall_clock64();
 
     // ---- phase 0: gate. Workgroup 0 also resets this launch's tickets and readiness counters;
     // nothing reads them before the second barrier.
     if (blockIdx.x == 0) {
         for (uint32_t i = tid; i < kXcds + p.E * mt_max; i += kThreads) sched[kSchedTicket + i] = 0u;
     }
-    for (uint32_t tile = blockIdx.x; tile < p.n_gate_tiles; tile += nwg)
-        gate_tile<T, NG>(p, tile, reinterpret_cast<float*>(smem));
+    for (uint32_t t0 = blockIdx.x * kGroups; t0 < p.n_gate_tiles; t0 += nwg * kGroups)
+        gate_tile<T, NG>(p, t0 + group, t0 + group < p.n_gate_tiles,
+                         reinterpret_cast<float*>(smem) + group * gate_smem_floats<NG>());
+    if (tid == 0) stamp[1] = wall_clock64();
     grid_barrier(sched, 0, barrier_base + nwg);
+    if (tid == 0) stamp[2] = wall_clock64();
 
     // ---- phase 1: slots in token order
     {
         uint32_t* base = reinterpret_cast<uint32_t*>(smem) + wave * p.E;
-        for (uint32_t t0 = blockIdx.x * 4; t0 < p.n_gate_tiles; t0 += nwg * 4)
+        for (uint32_t t0 = blockIdx.x * kWaves; t0 < p.n_gate_tiles; t0 += nwg * kWaves)
             slot_tile(p, t0 + wave, t0 + wave < p.n_gate_tiles, base);
         uint32_t* other = p.super_count + size_t((p.epoch & 1u) ^ 1u) * p.n_super * p.E;
         for (uint32_t i = blockIdx.x * kThreads + tid; i < p.n_super * p.E; i += nwg * kThreads) other[i] = 0u;
     }
+    if (tid == 0) stamp[3] = wall_clock64();
     grid_barrier(sched, 1, barrier_base + nwg);
+    if (tid == 0) stamp[4] = wall_clock64();
 
     // ---- phase 2: expert tiles from per-XCD ticket queues
     // LDS map: row blocks per expert | queue starts, totals, task | segments | GEMM tile
     uint16_t* s_mt = reinterpret_cast<uint16_t*>(smem);                         // [E], E <= 256
     uint32_t* s_qseg = reinterpret_cast<uint32_t*>(smem + kLdsMt);              // [9] first segment of each queue
     uint32_t* s_qtot = s_qseg + 16;                                             // [8] tickets in each queue
-    uint32_t* s_task = s_qtot + 8;                                              // [4] expert, kind, mtile, ntile (kind 2 = stop)
+    uint32_t* s_task = s_qtot + 8;                                              // [5] expert, kind, mtile, ntile, stolen (kind 2 = stop)
     Segment* s_seg = reinterpret_cast<Segment*>(smem + kLdsMt + kLdsQueue);     // at most 2*E segments
     char* s_gemm = smem + kFusedLdsHeader;
     const uint32_t tn_up = ceil_div_u32(p.I, BN), tn_down = ceil_div_u32(p.H, BN);
@@ -248,12 +261,16 @@ __global__ __launch_bounds__(kThreads) void fused_kernel(const LayerParams p, ui
     }
     __syncthreads();
 
+    // The XCD this workgroup really runs on (hardware register XCC_ID): expert e's tiles are queued
+    // on XCD e % 8, so that its weights, its gathered rows and the h1 rows handed from its
+    // up-projection to its down-projection all live in one L2.
+    const uint32_t xcd = __builtin_amdgcn_s_getreg((3 << 11) | 20) & (kXcds - 1);
     uint32_t q_off = 0;   // queues already found empty, starting from this workgroup's own XCD
     for (;;) {
         if (tid == 0) {
-            uint32_t kind = 2, e = 0, mtile = 0, ntile = 0;
+            uint32_t kind = 2, e = 0, mtile = 0, ntile = 0, stolen = 0;
             while (q_off < kXcds) {
-                const uint32_t q = (blockIdx.x + q_off) % kXcds;
+                const uint32_t q = (xcd + q_off) % kXcds;
                 // cheap pre-check keeps exhausted queues from being hammered
                 if (s_qtot[q] == 0) { ++q_off; continue; }
                 const uint32_t ticket = atomic_add_agent(sched + kSchedTicket + q, 1u);
@@ -266,6 +283,7 @@ __global__ __launch_bounds__(kThreads) void fused_kernel(const LayerParams p, ui
                 const uint32_t local = ticket - s_seg[s].start;
                 mtile = local % s_mt[e];
                 ntile = local / s_mt[e];
+                stolen = q_off != 0;
                 break;
             }
             if (kind == 1) {
@@ -273,12 +291,15 @@ __global__ __launch_bounds__(kThreads) void fused_kernel(const LayerParams p, ui
                 const uint32_t* ready = sched + kSchedReady + e * mt_max + mtile;
                 bounded_wait(sched, [&] { return atomic_load_relaxed(ready) >= tn_up; });
             }
-            s_task[0] = e; s_task[1] = kind; s_task[2] = mtile; s_task[3] = ntile;
+            s_task[0] = e; s_task[1] = kind; s_task[2] = mtile; s_task[3] = ntile; s_task[4] = stolen;
         }
         __syncthreads();
         const uint32_t e = s_task[0], kind = s_task[1], mtile = s_task[2], ntile = s_task[3];
         if (kind == 2) break;
-        if (kind == 1) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        // h1 rows written on this XCD are current in its L2 and the down-projection reads them
+        // past the L1; rows written on another XCD (a tile taken from a foreign queue) need the
+        // device-scope acquire, which drops this XCD's stale L2 lines.
+        if (kind == 1 && (s_task[4] || sizeof(T) != 2)) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
         expert_tile<T>(p, e, kind, mtile, ntile, kept_rows(p, e), s_gemm);
         __syncthreads();   // all stores of the tile issued; also protects s_task
         if (kind == 0 && tid == 0) {
@@ -286,17 +307,21 @@ __global__ __launch_bounds__(kThreads) void fused_kernel(const LayerParams p, ui
             atomic_add_agent(sched + kSchedReady + e * mt_max + mtile, 1u);
         }
     }
+    if (tid == 0) stamp[5] = wall_clock64();
     grid_barrier(sched, 2, barrier_base + nwg);
+    if (tid == 0) stamp[6] = wall_clock64();
 
     // ---- phase 3: combine, one token per wavefront
-    for (uint32_t token = blockIdx.x * 4 + wave; token < p.S; token += nwg * 4) combine_token<T>(p, token);
+    for (uint32_t token = blockIdx.x * kWaves + wave; token < p.S; token += nwg * kWaves) combine_token<T>(p, token);
+    __syncthreads();
+    if (tid == 0) stamp[7] = wall_clock64();
 }
 
 template <typename T, int NG>
 size_t fused_smem_bytes(uint32_t E) {
     size_t need = kFusedLdsHeader + gemm_smem_bytes<T>();
-    const size_t gate = gate_smem_floats<NG>() * sizeof(float);
-    const size_t slots = 4 * size_t(E) * sizeof(uint32_t);
+    const size_t gate = (TileShape<T>::kThreads / 256) * gate_smem_floats<NG>() * sizeof(float);
+    const size_t slots = (TileShape<T>::kThreads / kWave) * size_t(E) * sizeof(uint32_t);
     if (gate > need) need = gate;
     if (slots > need) need = slots;
     return need;
@@ -332,6 +357,12 @@ const char* unsupported_reason(uint32_t E, uint32_t k) {
 
 uint32_t sched_error_word() { return kSchedError; }
 
+#ifdef KLEOS_TRACE
+extern "C" int kleos_trace_attach(unsigned long long* device_buffer) {
+    return int(hipMemcpyToSymbol(HIP_SYMBOL(g_trace), &device_buffer, sizeof(device_buffer)));
+}
+#endif
+
 size_t sched_words(uint32_t E, uint32_t cap_rows) {
     return kSchedReady + size_t(E) * ceil_div_u32(cap_rows, 64) + 64;
 }
@@ -339,15 +370,15 @@ size_t sched_words(uint32_t E, uint32_t cap_rows) {
 hipError_t launch_gate(const LayerParams& p, int dtype, hipStream_t s) {
     return dispatch_groups(p.E, [&](auto ng) {
         constexpr int NG = decltype(ng)::value;
-        if (dtype == 2) hipLaunchKernelGGL((gate_kernel<bf16_t, NG>), dim3(p.n_gate_tiles), dim3(kThreads), 0, s, p);
-        else hipLaunchKernelGGL((gate_kernel<float, NG>), dim3(p.n_gate_tiles), dim3(kThreads), 0, s, p);
+        if (dtype == 2) hipLaunchKernelGGL((gate_kernel<bf16_t, NG>), dim3(p.n_gate_tiles), dim3(kPhaseThreads), 0, s, p);
+        else hipLaunchKernelGGL((gate_kernel<float, NG>), dim3(p.n_gate_tiles), dim3(kPhaseThreads), 0, s, p);
         return hipGetLastError();
     });
 }
 
 hipError_t launch_slots(const LayerParams& p, hipStream_t s) {
     const uint32_t grid = ceil_div_u32(p.n_gate_tiles, 4);
-    hipLaunchKernelGGL(slot_kernel, dim3(grid), dim3(kThreads), 4 * p.E * sizeof(uint32_t), s, p);
+    hipLaunchKernelGGL(slot_kernel, dim3(grid), dim3(kPhaseThreads), 4 * p.E * sizeof(uint32_t), s, p);
     return hipGetLastError();
 }
 
@@ -358,7 +389,12 @@ hipError_t launch_expert_gemm(const LayerParams& p, int dtype, int kind, hipStre
         const uint32_t cap = p.EC < p.cap_rows ? p.EC : p.cap_rows;
         const uint32_t tiles_m = ceil_div_u32(cap, TileShape<T>::BM), tiles_n = ceil_div_u32(N, TileShape<T>::BN);
         const uint32_t grid = p.E * tiles_m * tiles_n;
-        hipLaunchKernelGGL((expert_gemm_kernel<T>), dim3(grid), dim3(kThreads), gemm_smem_bytes<T>(), s, p,
+        auto kernel = expert_gemm_kernel<T>;
+        // more than 64 KB of dynamic LDS has to be asked for explicitly
+        hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, gemm_smem_bytes<T>());
+        if (err != hipSuccess) return err;
+        hipLaunchKernelGGL(kernel, dim3(grid), dim3(TileShape<T>::kThreads), gemm_smem_bytes<T>(), s, p,
                            uint32_t(kind), tiles_m, tiles_n);
         return hipGetLastError();
     };
@@ -367,8 +403,8 @@ hipError_t launch_expert_gemm(const LayerParams& p, int dtype, int kind, hipStre
 
 hipError_t launch_combine(const LayerParams& p, int dtype, hipStream_t s) {
     const uint32_t grid = ceil_div_u32(p.S, 4);
-    if (dtype == 2) hipLaunchKernelGGL((combine_kernel<bf16_t>), dim3(grid), dim3(kThreads), 0, s, p);
-    else hipLaunchKernelGGL((combine_kernel<float>), dim3(grid), dim3(kThreads), 0, s, p);
+    if (dtype == 2) hipLaunchKernelGGL((combine_kernel<bf16_t>), dim3(grid), dim3(kPhaseThreads), 0, s, p);
+    else hipLaunchKernelGGL((combine_kernel<float>), dim3(grid), dim3(kPhaseThreads), 0, s, p);
     return hipGetLastError();
 }
 
@@ -383,7 +419,7 @@ hipError_t plan_fused(const LayerParams& p, int dtype, int num_cus, FusedPlan* p
                                                  hipFuncAttributeMaxDynamicSharedMemorySize, int(smem));
             if (err != hipSuccess) return err;
             int occ = 0;
-            err = hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, kernel, kThreads, smem);
+            err = hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, kernel, TileShape<T>::kThreads, smem);
             if (err != hipSuccess) return err;
             if (occ < 1) return hipErrorLaunchOutOfResources;
             if (occ > 2) occ = 2;
@@ -398,6 +434,7 @@ hipError_t plan_fused(const LayerParams& p, int dtype, int num_cus, FusedPlan* p
             plan->lag = ceil_div_u32(ceil_div_u32(plan->nwg, kXcds), tiles_per_expert ? tiles_per_expert : 1u);
             if (plan->lag < 1) plan->lag = 1;
             plan->kernel = reinterpret_cast<const void*>(kernel);
+            plan->threads = TileShape<T>::kThreads;
             return hipSuccess;
         };
         return dtype == 2 ? go(bf16_t{}) : go(float{});
@@ -410,7 +447,7 @@ hipError_t launch_fused(const LayerParams& p, const FusedPlan& plan, uint32_t fu
     uint32_t mt_max = plan.mt_max, lag = plan.lag;
     LayerParams pc = p;
     void* args[] = {&pc, &barrier_base, &mt_max, &lag};
-    return hipLaunchKernel(plan.kernel, dim3(plan.nwg), dim3(kThreads), args, plan.smem, s);
+    return hipLaunchKernel(plan.kernel, dim3(plan.nwg), dim3(plan.threads), args, plan.smem, s);
 }
 
 }  // namespace kleos_amd

@@ -22,6 +22,7 @@ hipError_t launch_combine(const LayerParams& p, int dtype, hipStream_t s);
 struct FusedPlan {
     const void* kernel = nullptr;
     uint32_t nwg = 0;
+    uint32_t threads = 0;
     size_t smem = 0;
     uint32_t mt_max = 0;   // row blocks per expert at full capacity
     uint32_t lag = 0;      // experts between an up-projection segment and its down-projection segment

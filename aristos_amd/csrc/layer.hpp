@@ -45,7 +45,8 @@ struct LayerParams {
     void* h1;                 // [E][cap_rows, I]
     void* y;                  // [E][cap_rows, H]
     // ---- scheduler state of the persistent kernel
-    uint32_t* sched;          // counters, see scheduler section of moe_kernels.hip
+    uint32_t* sched;          // counters, see the scheduler section of kernels.hip
+    unsigned long long* stamps;   // [workgroups][8] 100 MHz wall-clock stamps of the phase boundaries
     uint32_t epoch;           // launch parity, selects the live half of double-buffered counters
 };
 

@@ -158,9 +158,12 @@ int kleos_moe_debug_views(kleos_debug_views_t* views);
  * any device buffer) into host memory. A convenience for callers without a HIP runtime binding. */
 int kleos_debug_copy_to_host(void* host_dst, const void* device_src, size_t bytes);
 
-/* Per-phase device time of the most recent kleos_moe_forward_bench in KLEOS_MODE_PHASED, in
- * milliseconds per launch: [0] gate, [1] slotting, [2] up-projection, [3] down-projection,
- * [4] combine. Zero-filled in fused mode. */
+/* Per-phase device time of the most recent kleos_moe_forward_bench, in milliseconds per launch:
+ * [0] gate, [1] slotting, [2] up-projection, [3] down-projection, [4] combine.
+ * KLEOS_MODE_PHASED: event-timed kernels, averaged over the trials. KLEOS_MODE_FUSED: taken from
+ * wall-clock stamps every workgroup of the last persistent launch leaves at its phase boundaries
+ * (each phase through the grid barrier that ends it); the two projections interleave in one phase,
+ * reported in [2] with [3] = 0. */
 int kleos_phase_times(float ms[5]);
 
 /* ---- errors --------------------------------------------------------------------------------- */
