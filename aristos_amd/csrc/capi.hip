@@ -29,6 +29,7 @@ struct Context {
     uint32_t fused_seq = 0;         // fused forwards issued (grid-barrier arrival base)
     int mode = KLEOS_MODE_FUSED;
     float phase_ms[5] = {0, 0, 0, 0, 0};
+    double sched_stats[6] = {0, 0, 0, 0, 0, 0};
 };
 
 Context* g_ctx = nullptr;   // one context per process, like the reference's global state
@@ -61,7 +62,7 @@ ArenaLayout layout_arena(const kleos_config_t& c, uint32_t n_tiles, uint32_t n_s
     L.super_count = take(2 * size_t(n_super) * E * 4);
     L.sched = take(sched_words(c.E, c.cap_rows) * 4);
     L.expert_count = take(E * 4);
-    L.stamps = take(size_t(kMaxWorkgroups) * 8 * 8);
+    L.stamps = take(size_t(kMaxWorkgroups) * 16 * 8);
     L.zero_end = off;
     L.logits = take(S * E * 4);
     L.topk_expert = take(S * k * 4);
@@ -129,9 +130,9 @@ int enqueue_forward(Context& c, const void* iP, void* oP, hipEvent_t* ev) {
     if (ev) KLEOS_HIP(hipEventRecord(ev[1], c.stream));
     KLEOS_HIP(launch_slots(p, c.stream));
     if (ev) KLEOS_HIP(hipEventRecord(ev[2], c.stream));
-    KLEOS_HIP(launch_expert_gemm(p, dt, 0, c.stream));
+    KLEOS_HIP(launch_expert_gemm(p, dt, 0, c.num_cus, c.stream));
     if (ev) KLEOS_HIP(hipEventRecord(ev[3], c.stream));
-    KLEOS_HIP(launch_expert_gemm(p, dt, 1, c.stream));
+    KLEOS_HIP(launch_expert_gemm(p, dt, 1, c.num_cus, c.stream));
     if (ev) KLEOS_HIP(hipEventRecord(ev[4], c.stream));
     KLEOS_HIP(launch_combine(p, dt, c.stream));
     if (ev) KLEOS_HIP(hipEventRecord(ev[5], c.stream));
@@ -292,13 +293,16 @@ extern "C" int kleos_moe_forward_bench(const void* iP, void* oP, uint32_t skip, 
         for (float& v : c.phase_ms) v = 0.f;
         if (!phased) {
             // phase boundaries of the last launch, stamped by every workgroup of the persistent kernel
-            std::vector<unsigned long long> st(size_t(c.plan.nwg) * 8);
+            std::vector<unsigned long long> st(size_t(c.plan.nwg) * 16);
             KLEOS_HIP(hipMemcpy(st.data(), c.base.stamps, st.size() * 8, hipMemcpyDeviceToHost));
             unsigned long long t0 = ~0ull, b[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+            for (int i = 0; i < 6; ++i) c.sched_stats[i] = 0.0;
             for (uint32_t w = 0; w < c.plan.nwg; ++w) {
-                t0 = std::min(t0, st[size_t(w) * 8]);
-                for (int i = 0; i < 8; ++i) b[i] = std::max(b[i], st[size_t(w) * 8 + i]);
+                t0 = std::min(t0, st[size_t(w) * 16]);
+                for (int i = 0; i < 8; ++i) b[i] = std::max(b[i], st[size_t(w) * 16 + i]);
+                for (int i = 0; i < 6; ++i) c.sched_stats[i] += double(st[size_t(w) * 16 + 8 + i]);
             }
+            for (int i = 0; i < 3; ++i) c.sched_stats[i] *= 1e-5 / double(c.plan.nwg);   // mean ms per workgroup
             const float tick_ms = 1e-5f;   // 100 MHz
             c.phase_ms[0] = float(b[2] - t0) * tick_ms;        // gate, through the first grid barrier
             c.phase_ms[1] = float(b[4] - b[2]) * tick_ms;      // slots, through the second
@@ -351,6 +355,13 @@ extern "C" int kleos_debug_copy_to_host(void* host_dst, const void* device_src, 
     if (!host_dst || !device_src) return fail(KLEOS_EINVAL, "kleos_debug_copy_to_host: null argument");
     KLEOS_HIP(hipStreamSynchronize(g_ctx->stream));
     KLEOS_HIP(hipMemcpy(host_dst, device_src, bytes, hipMemcpyDeviceToHost));
+    return KLEOS_OK;
+}
+
+extern "C" int kleos_scheduler_stats(double stats[6]) {
+    if (int rc = require_ctx("kleos_scheduler_stats")) return rc;
+    if (!stats) return fail(KLEOS_EINVAL, "kleos_scheduler_stats: null argument");
+    for (int i = 0; i < 6; ++i) stats[i] = g_ctx->sched_stats[i];
     return KLEOS_OK;
 }
 

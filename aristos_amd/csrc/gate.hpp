@@ -55,7 +55,25 @@ __device__ __forceinline__ void gate_tile(const LayerParams& p, uint32_t tile, b
     for (int g = 0; g < NG; ++g) acc[g] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     // logits^T tile: experts are the matrix-core rows, tokens its columns (gate.cuh:526-534).
-    for (uint32_t s = valid ? s0 : s1; s < s1; ++s) {
+    // The loads of U steps are issued together before their matrix instructions: the activation
+    // rows stream from HBM once and this is what keeps enough of them in flight.
+    constexpr int U = NG <= 4 ? 4 : (NG <= 8 ? 2 : 1);
+    uint32_t s = valid ? s0 : s1;
+    for (; s + U <= s1; s += U) {
+        u32x4 b[U], a[U][NG];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const uint32_t off = (s + u) * kStepK;
+            b[u] = load16(xrow + off);
+#pragma unroll
+            for (int g = 0; g < NG; ++g) a[u][g] = load16(wrow + size_t(g) * 16 * H + off);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int g = 0; g < NG; ++g) acc[g] = mma16_step(a[u][g], b[u], acc[g], T{});
+    }
+    for (; s < s1; ++s) {
         const uint32_t off = s * kStepK;
         const u32x4 b = load16(xrow + off);
 #pragma unroll

@@ -26,22 +26,27 @@ namespace {
 
 constexpr int kXcds = 8;
 // expert GEMM tile of the bf16 path
+// Expert GEMM configuration of the bf16 path: 256 x 256 tile (an expert's whole capacity of 256 rows
+// at the headline shape, so its weights stream from HBM exactly once), 2 x 4 wavefronts of 128 x 64
+// (two per SIMD), K slices of 64 (whole 128-byte lines of every row) through two 64 KB stages.
+using GemmCfg = GemmBf16<256, 256, 2, 4, 64, 2>;
 constexpr int kBM = 256, kBN = 256;
-constexpr int kWavesM = 2, kWavesN = 4;   // wavefront grid over the tile
-constexpr int kGemmThreads = kWavesM * kWavesN * kWave;
+constexpr int kGemmThreads = GemmCfg::kThreads;
 
 // Tile shape and workgroup size of the expert projections per Element type. The workgroup size is
 // also that of the persistent kernel, whose other phases run on groups of its wavefronts.
 template <typename T> struct TileShape;
-template <> struct TileShape<bf16_t> { static constexpr int BM = kBM, BN = kBN, kThreads = kGemmThreads; };
-template <> struct TileShape<float> { static constexpr int BM = kF32Tile, BN = kF32Tile, kThreads = 256; };
+template <> struct TileShape<bf16_t> { static constexpr int BM = kBM, BN = kBN, kThreads = kGemmThreads, kPerCu = 1; };
+template <> struct TileShape<float> { static constexpr int BM = kF32Tile, BN = kF32Tile, kThreads = 256, kPerCu = 1; };
 constexpr int kPhaseThreads = 256;   // gate, slot and combine kernels of the phased mode
 
 template <typename T>
 constexpr int gemm_smem_bytes() {
-    if constexpr (sizeof(T) == 2) return gemm_bf16_smem_bytes<kBM, kBN>();
+    if constexpr (sizeof(T) == 2) return GemmCfg::kSmemBytes;
     else return gemm_f32_smem_bytes();
 }
+constexpr int kPhasedGemmHeader = 128;
+constexpr int kStampWords = 16;         // per-workgroup phase stamps [0..7] and scheduler statistics [8..15]   // task broadcast slot in front of the GEMM stages
 
 __host__ __device__ inline uint32_t ceil_div_u32(uint32_t a, uint32_t b) { return (a + b - 1) / b; }
 
@@ -52,92 +57,7 @@ __device__ __forceinline__ uint32_t kept_rows(const LayerParams& p, uint32_t e) 
     return c < cap ? c : cap;
 }
 
-// One output tile of an expert projection. kind 0: h1 = act(x_gathered * Wup^T + bup);
-// kind 1: y = h1 * Wdown^T + bdown (identity activation, types.cuh:461).
-template <typename T>
-__device__ __forceinline__ void expert_tile(const LayerParams& p, uint32_t e, uint32_t kind,
-                                            uint32_t mtile, uint32_t ntile, uint32_t rows,
-                                            char* smem) {
-    constexpr int BM = TileShape<T>::BM, BN = TileShape<T>::BN;
-    const uint32_t row0 = mtile * BM, col0 = ntile * BN;
-    const uint32_t m_valid = rows - row0 < uint32_t(BM) ? rows - row0 : uint32_t(BM);
-    const uint32_t N = kind == 0 ? p.I : p.H, K = kind == 0 ? p.H : p.I;
-    const uint32_t n_valid = N - col0 < uint32_t(BN) ? N - col0 : uint32_t(BN);
-    const T* w = static_cast<const T*>(kind == 0 ? p.w_up : p.w_down) + size_t(e) * p.I * p.H + size_t(col0) * K;
-    const T* bias = static_cast<const T*>(kind == 0 ? p.b_up : p.b_down) + size_t(e) * N + col0;
-    const size_t row_base = size_t(e) * p.cap_rows + row0;
-    if (kind == 0) {
-        const T* a = static_cast<const T*>(p.x);
-        const int32_t* idx = p.slot_token + row_base;
-        T* c = static_cast<T*>(p.h1) + row_base * p.I + col0;
-        auto run = [&](auto act_tag) {
-            constexpr int ACT = decltype(act_tag)::value;
-            if constexpr (sizeof(T) == 2)
-                gemm_tile_bf16<ACT, BM, BN, kWavesM, kWavesN, 0>(a, idx, p.H, m_valid, w, K, n_valid, bias, c, p.I, K, smem);
-            else
-                gemm_tile_f32<ACT>(a, idx, p.H, m_valid, w, K, n_valid, bias, c, p.I, K, smem);
-        };
-        if (p.act == 0) run(std::integral_constant<int, 0>{});
-        else run(std::integral_constant<int, 1>{});
-    } else {
-        const T* a = static_cast<const T*>(p.h1) + row_base * p.I;
-        T* c = static_cast<T*>(p.y) + row_base * p.H + col0;
-        if constexpr (sizeof(T) == 2)
-            gemm_tile_bf16<2, BM, BN, kWavesM, kWavesN, 1>(a, nullptr, p.I, m_valid, w, K, n_valid, bias, c, p.H, K, smem);
-        else
-            gemm_tile_f32<2>(a, nullptr, p.I, m_valid, w, K, n_valid, bias, c, p.H, K, smem);
-    }
-}
-
-// ------------------------------------------------------------------------------------ phased
-template <typename T, int NG>
-__global__ __launch_bounds__(kPhaseThreads) void gate_kernel(const LayerParams p) {
-    __shared__ float smem[gate_smem_floats<NG>()];
-    gate_tile<T, NG>(p, blockIdx.x, true, smem);
-}
-
-__global__ __launch_bounds__(kPhaseThreads) void slot_kernel(const LayerParams p) {
-    extern __shared__ uint32_t slot_smem[];
-    const uint32_t wave = threadIdx.x >> 6;
-    const uint32_t tile = blockIdx.x * 4 + wave;
-    slot_tile(p, tile, tile < p.n_gate_tiles, slot_smem + wave * p.E);
-    // the coarse counts of the other epoch are free now: clear them for the next launch
-    uint32_t* other = p.super_count + size_t((p.epoch & 1u) ^ 1u) * p.n_super * p.E;
-    for (uint32_t i = blockIdx.x * kPhaseThreads + threadIdx.x; i < p.n_super * p.E; i += gridDim.x * kPhaseThreads)
-        other[i] = 0u;
-}
-
-// Workgroup -> (expert, row block, column block). Consecutive workgroup ids land on consecutive
-// XCDs, so expert e is pinned to XCD e % 8: all tiles that share its weights and its activation
-// rows meet in one L2. Row blocks vary fastest so that the tiles re-reading one weight tile run
-// together.
-template <typename T>
-__global__ __launch_bounds__(TileShape<T>::kThreads) void expert_gemm_kernel(const LayerParams p, uint32_t kind,
-                                                               uint32_t tiles_m, uint32_t tiles_n) {
-    extern __shared__ __attribute__((aligned(16))) char gemm_smem[];
-    const uint32_t per_expert = tiles_m * tiles_n;
-    uint32_t e, rem;
-    if (p.E % kXcds == 0) {
-        const uint32_t xcd = blockIdx.x % kXcds, j = blockIdx.x / kXcds;
-        e = xcd + kXcds * (j / per_expert);
-        rem = j % per_expert;
-    } else {
-        e = blockIdx.x / per_expert;
-        rem = blockIdx.x % per_expert;
-    }
-    const uint32_t mtile = rem % tiles_m, ntile = rem / tiles_m;
-    const uint32_t rows = kept_rows(p, e);
-    if (mtile * TileShape<T>::BM >= rows) return;
-    expert_tile<T>(p, e, kind, mtile, ntile, rows, gemm_smem);
-}
-
-template <typename T>
-__global__ __launch_bounds__(kPhaseThreads) void combine_kernel(const LayerParams p) {
-    const uint32_t token = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (token < p.S) combine_token<T>(p, token);
-}
-
-// ------------------------------------------------------------------------------------ fused
+// ------------------------------------------------------------------------------------ scheduler state
 // Scheduler words (uint32), all in p.sched:
 //   [0..2]                 grid-barrier arrival counters, monotonically increasing across launches
 //   [8..15]                ticket counter of each XCD queue
@@ -184,8 +104,238 @@ __device__ __forceinline__ void grid_barrier(uint32_t* sched, uint32_t which, ui
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
 }
 
+// One unit of expert work: an output tile of the up-projection (kind 0: h1 = act(x_gathered *
+// Wup^T + bup)) or of the down-projection (kind 1: y = h1 * Wdown^T + bdown, identity activation,
+// types.cuh:461). The reference's 128-byte Task descriptor (types.cuh:565-654) shrinks to this.
+struct Task {
+    uint32_t e, kind, mtile, ntile;
+    uint32_t foreign;   // taken from another XCD's queue: its h1 rows may sit in a different L2
+    uint32_t ready;     // down tile whose up-projection row block was already complete when handed out
+    uint32_t valid;
+};
+constexpr int kTaskWords = 8;
+
+// Thread 0 publishes a task through LDS; every thread of the workgroup returns the same task.
+// The barrier inside also separates the caller's previous and next use of the LDS.
+__device__ __forceinline__ Task broadcast_task(uint32_t* s_task, const Task& mine) {
+    if (threadIdx.x == 0) {
+        s_task[0] = mine.e; s_task[1] = mine.kind; s_task[2] = mine.mtile; s_task[3] = mine.ntile;
+        s_task[4] = mine.foreign; s_task[5] = mine.ready; s_task[6] = mine.valid;
+    }
+    __syncthreads();
+    Task t;
+    t.e = s_task[0]; t.kind = s_task[1]; t.mtile = s_task[2]; t.ntile = s_task[3];
+    t.foreign = s_task[4]; t.ready = s_task[5]; t.valid = s_task[6];
+    return t;
+}
+
+template <typename T>
+struct TileOperands {
+    const T* a; const int32_t* idx; const T* w; const T* bias; T* c;
+    uint32_t lda, ldc, K, m_valid, n_valid, act;
+};
+
+template <typename T>
+__device__ __forceinline__ TileOperands<T> tile_operands(const LayerParams& p, const Task& t) {
+    constexpr int BM = TileShape<T>::BM, BN = TileShape<T>::BN;
+    TileOperands<T> o;
+    const uint32_t rows = kept_rows(p, t.e);
+    const uint32_t row0 = t.mtile * BM, col0 = t.ntile * BN;
+    const uint32_t N = t.kind == 0 ? p.I : p.H;
+    o.K = t.kind == 0 ? p.H : p.I;
+    o.m_valid = rows - row0 < uint32_t(BM) ? rows - row0 : uint32_t(BM);
+    o.n_valid = N - col0 < uint32_t(BN) ? N - col0 : uint32_t(BN);
+    o.w = static_cast<const T*>(t.kind == 0 ? p.w_up : p.w_down) + size_t(t.e) * p.I * p.H + size_t(col0) * o.K;
+    o.bias = static_cast<const T*>(t.kind == 0 ? p.b_up : p.b_down) + size_t(t.e) * N + col0;
+    const size_t row_base = size_t(t.e) * p.cap_rows + row0;
+    if (t.kind == 0) {
+        o.a = static_cast<const T*>(p.x); o.idx = p.slot_token + row_base; o.lda = p.H;
+        o.c = static_cast<T*>(p.h1) + row_base * p.I + col0; o.ldc = p.I; o.act = p.act;
+    } else {
+        o.a = static_cast<const T*>(p.h1) + row_base * p.I; o.idx = nullptr; o.lda = p.I;
+        o.c = static_cast<T*>(p.y) + row_base * p.H + col0; o.ldc = p.H; o.act = 2;
+    }
+    return o;
+}
+
+// Readiness of a down-projection tile: all up-projection tiles of its (expert, row block) stored.
+struct Readiness {
+    uint32_t* sched;      // nullptr: no cross-tile dependencies inside this launch (phased mode)
+    uint32_t mt_max, tn_up;
+    __device__ __forceinline__ uint32_t* counter(const Task& t) const { return sched + kSchedReady + t.e * mt_max + t.mtile; }
+};
+
+// The expert phase of one workgroup: tiles from `next` until it runs dry. `next()` is called by
+// every thread and returns the same task in all of them without ever blocking on a dependency;
+// blocking happens here, after the workgroup has published its own finished tile, so that two
+// workgroups can never wait on each other's unpublished results.
+// `stats` (thread 0 only, may be null) accumulates 100 MHz ticks spent [0] fetching tasks,
+// [1] waiting for a dependency, [2] publishing, and counts [3] tiles, [4] tiles handed out before
+// their inputs were complete, [5] tiles taken from a foreign queue.
+template <typename T, typename Next>
+__device__ __forceinline__ void expert_loop(const LayerParams& p, char* smem, uint32_t* s_task, const Readiness rd,
+                                            unsigned long long* stats, Next&& next_raw) {
+    const uint32_t tid = threadIdx.x;
+    unsigned long long st_next = 0, st_wait = 0, st_pub = 0, n_tiles = 0, n_late = 0, n_foreign = 0;
+    auto next = [&]() {
+        const unsigned long long t0 = wall_clock64();
+        const Task t = next_raw();
+        st_next += wall_clock64() - t0;
+        if (t.valid) { ++n_tiles; n_late += !t.ready; n_foreign += t.foreign; }
+        return t;
+    };
+    auto wait_ready = [&](const Task& t) {
+        // only a down tile handed out before its inputs were complete gets here
+        const unsigned long long t0 = wall_clock64();
+        if (tid == 0) bounded_wait(rd.sched, [&] { return atomic_load_relaxed(rd.counter(t)) >= rd.tn_up; });
+        __syncthreads();
+        st_wait += wall_clock64() - t0;
+    };
+    auto flush_stats = [&]() {
+        if (stats && tid == 0) {
+            stats[0] = st_next; stats[1] = st_wait; stats[2] = st_pub; stats[3] = n_tiles; stats[4] = n_late; stats[5] = n_foreign;
+        }
+    };
+    auto acquire = [&](const Task& t) {
+        // Before a down tile reads h1 rows that other workgroups of this launch wrote: rows written
+        // on this XCD are current in its L2, so dropping this CU's L1 is enough; rows written on
+        // another XCD need the device-scope acquire, which also drops this XCD's stale L2 lines.
+        if (!rd.sched || t.kind != 1) return;
+        if (t.foreign) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        else asm volatile("buffer_inv sc0" ::: "memory");
+    };
+    auto publish = [&](const Task& t) {
+        // all stores of the tile are complete in every wavefront; make them visible device-wide,
+        // then count the tile (the reference's tQS increment, processor.cuh:719)
+        if (rd.sched && t.kind == 0 && tid == 0) {
+            const unsigned long long t0 = wall_clock64();
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+            atomic_add_agent(rd.counter(t), 1u);
+            st_pub += wall_clock64() - t0;
+        }
+    };
+
+    if constexpr (sizeof(T) == 2) {
+        using G = GemmCfg;
+        auto args_of = [&](const Task& t) {
+            const TileOperands<T> o = tile_operands<T>(p, t);
+            GemmTileArgs g;
+            g.a_base = o.a; g.a_row_index = o.idx; g.b_base = o.w; g.bias = o.bias; g.c_base = o.c;
+            g.lda = o.lda; g.ldb = o.K; g.ldc = o.ldc; g.K = o.K; g.m_valid = o.m_valid; g.n_valid = o.n_valid;
+            g.act = o.act;
+            return g;
+        };
+        typename G::Tile cur_t, nxt_t;
+        typename G::Acc acc;
+        Task cur = next();
+        if (!cur.valid) { flush_stats(); return; }
+        if (cur.kind == 1 && !cur.ready) wait_ready(cur);
+        acquire(cur);
+        G::begin(cur_t, args_of(cur), 0, smem);
+        for (;;) {
+            G::mainloop(cur_t, acc, smem);
+                Task nxt = next();   // its barrier: every wavefront has left the main loop
+                const bool early = nxt.valid && (nxt.kind == 0 || nxt.ready);
+            if (early) {
+                // the next tile's index look-ups and first loads travel while this tile's epilogue runs
+                acquire(nxt);
+                G::begin(nxt_t, args_of(nxt), G::next_stage0(cur_t), smem);
+            }
+                G::finish(cur_t, acc, smem);
+                wait_vmcnt<0>();
+            __syncthreads();
+            publish(cur);
+                if (!nxt.valid) break;
+            if (!early) {
+                wait_ready(nxt);
+                acquire(nxt);
+                G::begin(nxt_t, args_of(nxt), G::next_stage0(cur_t), smem);
+            }
+            cur = nxt;
+            cur_t = nxt_t;
+        }
+        flush_stats();
+    } else {
+        for (;;) {
+            const Task t = next();
+            if (!t.valid) break;
+            if (t.kind == 1 && !t.ready) wait_ready(t);
+            acquire(t);
+            const TileOperands<T> o = tile_operands<T>(p, t);
+            if (o.act == 0) gemm_tile_f32<0>(o.a, o.idx, o.lda, o.m_valid, o.w, o.K, o.n_valid, o.bias, o.c, o.ldc, o.K, smem);
+            else if (o.act == 1) gemm_tile_f32<1>(o.a, o.idx, o.lda, o.m_valid, o.w, o.K, o.n_valid, o.bias, o.c, o.ldc, o.K, smem);
+            else gemm_tile_f32<2>(o.a, o.idx, o.lda, o.m_valid, o.w, o.K, o.n_valid, o.bias, o.c, o.ldc, o.K, smem);
+            __syncthreads();
+            publish(t);
+        }
+        flush_stats();
+    }
+}
+
+// ------------------------------------------------------------------------------------ phased
 template <typename T, int NG>
-__global__ __launch_bounds__(TileShape<T>::kThreads) void fused_kernel(const LayerParams p, uint32_t barrier_base,
+__global__ __launch_bounds__(kPhaseThreads) void gate_kernel(const LayerParams p) {
+    __shared__ float smem[gate_smem_floats<NG>()];
+    gate_tile<T, NG>(p, blockIdx.x, true, smem);
+}
+
+__global__ __launch_bounds__(kPhaseThreads) void slot_kernel(const LayerParams p) {
+    extern __shared__ uint32_t slot_smem[];
+    const uint32_t wave = threadIdx.x >> 6;
+    const uint32_t tile = blockIdx.x * 4 + wave;
+    slot_tile(p, tile, tile < p.n_gate_tiles, slot_smem + wave * p.E);
+    // the coarse counts of the other epoch are free now: clear them for the next launch
+    uint32_t* other = p.super_count + size_t((p.epoch & 1u) ^ 1u) * p.n_super * p.E;
+    for (uint32_t i = blockIdx.x * kPhaseThreads + threadIdx.x; i < p.n_super * p.E; i += gridDim.x * kPhaseThreads)
+        other[i] = 0u;
+}
+
+// One projection of every expert as a persistent grid with a static schedule: workgroup b takes
+// the tiles b, b + G, b + 2G, ... of the list (expert, column block, row block). Consecutive
+// workgroup ids land on consecutive XCDs, so with E a multiple of 8 expert e stays on XCD e % 8:
+// all tiles that share its weights and its activation rows meet in one L2. Row blocks vary
+// fastest so that the tiles re-reading one weight tile run together.
+template <typename T>
+__global__ __launch_bounds__(TileShape<T>::kThreads, TileShape<T>::kPerCu) void expert_gemm_kernel(const LayerParams p, uint32_t kind,
+                                                               uint32_t tiles_m, uint32_t tiles_n) {
+    extern __shared__ __attribute__((aligned(16))) char gemm_smem[];
+    uint32_t* s_task = reinterpret_cast<uint32_t*>(gemm_smem);
+    const uint32_t per_expert = tiles_m * tiles_n, total = p.E * per_expert;
+    uint32_t i = blockIdx.x;
+    auto next = [&]() {
+        Task t{};
+        if (threadIdx.x == 0) {
+            for (; i < total; i += gridDim.x) {
+                uint32_t e, rem;
+                if (p.E % kXcds == 0) {
+                    const uint32_t xcd = i % kXcds, j = i / kXcds;
+                    e = xcd + kXcds * (j / per_expert);
+                    rem = j % per_expert;
+                } else {
+                    e = i / per_expert;
+                    rem = i % per_expert;
+                }
+                const uint32_t mtile = rem % tiles_m;
+                if (mtile * TileShape<T>::BM >= kept_rows(p, e)) continue;   // the expert has fewer rows
+                t.e = e; t.kind = kind; t.mtile = mtile; t.ntile = rem / tiles_m; t.ready = 1; t.valid = 1;
+                i += gridDim.x;
+                break;
+            }
+        }
+        return broadcast_task(s_task, t);
+    };
+    expert_loop<T>(p, gemm_smem + kPhasedGemmHeader, s_task, Readiness{nullptr, 0, 0}, nullptr, next);
+}
+
+template <typename T>
+__global__ __launch_bounds__(kPhaseThreads) void combine_kernel(const LayerParams p) {
+    const uint32_t token = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (token < p.S) combine_token<T>(p, token);
+}
+
+// ------------------------------------------------------------------------------------ fused
+template <typename T, int NG>
+__global__ __launch_bounds__(TileShape<T>::kThreads, TileShape<T>::kPerCu) void fused_kernel(const LayerParams p, uint32_t barrier_base,
                                                                       uint32_t mt_max, uint32_t lag) {
     static_assert(sizeof(Segment) == 8, "segment table sizing");
     extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -195,7 +345,7 @@ __global__ __launch_bounds__(TileShape<T>::kThreads) void fused_kernel(const Lay
     const uint32_t tid = threadIdx.x, wave = tid >> 6, group = tid >> 8;
     const uint32_t nwg = gridDim.x;
     uint32_t* sched = p.sched;
-    unsigned long long* stamp = p.stamps + size_t(blockIdx.x) * 8;
+    unsigned long long* stamp = p.stamps + size_t(blockIdx.x) * kStampWords;
     if (tid == 0) stamp[0] = wall_clock64();
 
     // ---- phase 0: gate. Workgroup 0 also resets this launch's tickets and readiness counters;
@@ -227,7 +377,7 @@ __global__ __launch_bounds__(TileShape<T>::kThreads) void fused_kernel(const Lay
     uint16_t* s_mt = reinterpret_cast<uint16_t*>(smem);                         // [E], E <= 256
     uint32_t* s_qseg = reinterpret_cast<uint32_t*>(smem + kLdsMt);              // [9] first segment of each queue
     uint32_t* s_qtot = s_qseg + 16;                                             // [8] tickets in each queue
-    uint32_t* s_task = s_qtot + 8;                                              // [5] expert, kind, mtile, ntile, stolen (kind 2 = stop)
+    uint32_t* s_task = s_qtot + 8;                                              // [kTaskWords] task broadcast slot
     Segment* s_seg = reinterpret_cast<Segment*>(smem + kLdsMt + kLdsQueue);     // at most 2*E segments
     char* s_gemm = smem + kFusedLdsHeader;
     const uint32_t tn_up = ceil_div_u32(p.I, BN), tn_down = ceil_div_u32(p.H, BN);
@@ -266,47 +416,33 @@ __global__ __launch_bounds__(TileShape<T>::kThreads) void fused_kernel(const Lay
     // up-projection to its down-projection all live in one L2.
     const uint32_t xcd = __builtin_amdgcn_s_getreg((3 << 11) | 20) & (kXcds - 1);
     uint32_t q_off = 0;   // queues already found empty, starting from this workgroup's own XCD
-    for (;;) {
+    const Readiness rd{sched, mt_max, tn_up};
+    auto next = [&]() {
+        Task t{};
         if (tid == 0) {
-            uint32_t kind = 2, e = 0, mtile = 0, ntile = 0, stolen = 0;
             while (q_off < kXcds) {
                 const uint32_t q = (xcd + q_off) % kXcds;
                 // cheap pre-check keeps exhausted queues from being hammered
                 if (s_qtot[q] == 0) { ++q_off; continue; }
                 const uint32_t ticket = atomic_add_agent(sched + kSchedTicket + q, 1u);
                 if (ticket >= s_qtot[q]) { ++q_off; continue; }
-                uint32_t s = s_qseg[q];
-                const uint32_t s_end = s_qseg[q + 1];
-                while (s + 1 < s_end && s_seg[s + 1].start <= ticket) ++s;
-                e = s_seg[s].expert;
-                kind = s_seg[s].kind;
-                const uint32_t local = ticket - s_seg[s].start;
-                mtile = local % s_mt[e];
-                ntile = local / s_mt[e];
-                stolen = q_off != 0;
+                uint32_t sg = s_qseg[q];
+                const uint32_t sg_end = s_qseg[q + 1];
+                while (sg + 1 < sg_end && s_seg[sg + 1].start <= ticket) ++sg;
+                t.e = s_seg[sg].expert;
+                t.kind = s_seg[sg].kind;
+                const uint32_t local = ticket - s_seg[sg].start;
+                t.mtile = local % s_mt[t.e];
+                t.ntile = local / s_mt[t.e];
+                t.foreign = q_off != 0;
+                t.ready = t.kind == 0 || atomic_load_relaxed(rd.counter(t)) >= tn_up;
+                t.valid = 1;
                 break;
             }
-            if (kind == 1) {
-                // wait until every up-projection tile of this row block is stored
-                const uint32_t* ready = sched + kSchedReady + e * mt_max + mtile;
-                bounded_wait(sched, [&] { return atomic_load_relaxed(ready) >= tn_up; });
-            }
-            s_task[0] = e; s_task[1] = kind; s_task[2] = mtile; s_task[3] = ntile; s_task[4] = stolen;
         }
-        __syncthreads();
-        const uint32_t e = s_task[0], kind = s_task[1], mtile = s_task[2], ntile = s_task[3];
-        if (kind == 2) break;
-        // h1 rows written on this XCD are current in its L2 and the down-projection reads them
-        // past the L1; rows written on another XCD (a tile taken from a foreign queue) need the
-        // device-scope acquire, which drops this XCD's stale L2 lines.
-        if (kind == 1 && (s_task[4] || sizeof(T) != 2)) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-        expert_tile<T>(p, e, kind, mtile, ntile, kept_rows(p, e), s_gemm);
-        __syncthreads();   // all stores of the tile issued; also protects s_task
-        if (kind == 0 && tid == 0) {
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-            atomic_add_agent(sched + kSchedReady + e * mt_max + mtile, 1u);
-        }
-    }
+        return broadcast_task(s_task, t);
+    };
+    expert_loop<T>(p, s_gemm, s_task, rd, stamp + 8, next);
     if (tid == 0) stamp[5] = wall_clock64();
     grid_barrier(sched, 2, barrier_base + nwg);
     if (tid == 0) stamp[6] = wall_clock64();
@@ -357,11 +493,6 @@ const char* unsupported_reason(uint32_t E, uint32_t k) {
 
 uint32_t sched_error_word() { return kSchedError; }
 
-#ifdef KLEOS_TRACE
-extern "C" int kleos_trace_attach(unsigned long long* device_buffer) {
-    return int(hipMemcpyToSymbol(HIP_SYMBOL(g_trace), &device_buffer, sizeof(device_buffer)));
-}
-#endif
 
 size_t sched_words(uint32_t E, uint32_t cap_rows) {
     return kSchedReady + size_t(E) * ceil_div_u32(cap_rows, 64) + 64;
@@ -382,20 +513,31 @@ hipError_t launch_slots(const LayerParams& p, hipStream_t s) {
     return hipGetLastError();
 }
 
-hipError_t launch_expert_gemm(const LayerParams& p, int dtype, int kind, hipStream_t s) {
+hipError_t launch_expert_gemm(const LayerParams& p, int dtype, int kind, int num_cus, hipStream_t s) {
     const uint32_t N = kind == 0 ? p.I : p.H;
     auto go = [&](auto tag) {
         using T = decltype(tag);
         const uint32_t cap = p.EC < p.cap_rows ? p.EC : p.cap_rows;
         const uint32_t tiles_m = ceil_div_u32(cap, TileShape<T>::BM), tiles_n = ceil_div_u32(N, TileShape<T>::BN);
-        const uint32_t grid = p.E * tiles_m * tiles_n;
+        const uint32_t total = p.E * tiles_m * tiles_n;
         auto kernel = expert_gemm_kernel<T>;
-        // more than 64 KB of dynamic LDS has to be asked for explicitly
-        hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                             hipFuncAttributeMaxDynamicSharedMemorySize, gemm_smem_bytes<T>());
-        if (err != hipSuccess) return err;
-        hipLaunchKernelGGL(kernel, dim3(grid), dim3(TileShape<T>::kThreads), gemm_smem_bytes<T>(), s, p,
-                           uint32_t(kind), tiles_m, tiles_n);
+        constexpr int smem = kPhasedGemmHeader + gemm_smem_bytes<T>();
+        static int resident = 0;   // workgroups per CU, found once per Element type
+        if (resident == 0) {
+            // more than 64 KB of dynamic LDS has to be asked for explicitly
+            hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+            if (err != hipSuccess) return err;
+            int occ = 0;
+            err = hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, kernel, TileShape<T>::kThreads, smem);
+            if (err != hipSuccess) return err;
+            if (occ < 1) return hipErrorLaunchOutOfResources;
+            resident = occ;
+        }
+        // persistent grid: as many workgroups as stay resident, a multiple of the XCD count
+        uint32_t grid = uint32_t(num_cus) * uint32_t(resident);
+        if (grid > total) grid = (total + kXcds - 1) / kXcds * kXcds;
+        hipLaunchKernelGGL(kernel, dim3(grid), dim3(TileShape<T>::kThreads), smem, s, p, uint32_t(kind), tiles_m, tiles_n);
         return hipGetLastError();
     };
     return dtype == 2 ? go(bf16_t{}) : go(float{});

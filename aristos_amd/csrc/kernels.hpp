@@ -14,7 +14,7 @@ uint32_t sched_error_word();
 // Phase launchers (KLEOS_MODE_PHASED). dtype: 0 fp32, 2 bf16.
 hipError_t launch_gate(const LayerParams& p, int dtype, hipStream_t s);
 hipError_t launch_slots(const LayerParams& p, hipStream_t s);
-hipError_t launch_expert_gemm(const LayerParams& p, int dtype, int kind /*0 up, 1 down*/, hipStream_t s);
+hipError_t launch_expert_gemm(const LayerParams& p, int dtype, int kind /*0 up, 1 down*/, int num_cus, hipStream_t s);
 hipError_t launch_combine(const LayerParams& p, int dtype, hipStream_t s);
 
 // The whole layer as one persistent launch (KLEOS_MODE_FUSED). The plan fixes the grid (every

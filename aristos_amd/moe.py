@@ -48,6 +48,14 @@ def phase_times() -> dict:
     return dict(zip(("gate", "slots", "up", "down", "combine"), (float(v) for v in arr)))
 
 
+def scheduler_stats() -> dict:
+    """Tile-scheduler statistics of the last fused forward_host_bench launch."""
+    arr = (C.c_double * 6)()
+    _capi.check(_capi.lib().kleos_scheduler_stats(arr))
+    keys = ("fetch_ms", "wait_ms", "publish_ms", "tiles", "late_tiles", "foreign_tiles")
+    return dict(zip(keys, (float(v) for v in arr)))
+
+
 def debug_views(derived) -> dict:
     """Copies the routing state of the most recent forward to host numpy arrays. Synchronises."""
     lib = _capi.lib()

@@ -165,6 +165,12 @@ int kleos_debug_copy_to_host(void* host_dst, const void* device_src, size_t byte
  * (each phase through the grid barrier that ends it); the two projections interleave in one phase,
  * reported in [2] with [3] = 0. */
 int kleos_phase_times(float ms[5]);
+/* Tile-scheduler statistics of the last launch of the most recent kleos_moe_forward_bench in
+ * KLEOS_MODE_FUSED (the persistent kernel keeps them per workgroup; the reference has no
+ * counterpart): [0..2] mean milliseconds a workgroup spent fetching tasks, waiting for an
+ * unfinished dependency, publishing finished tiles; [3] expert tiles executed; [4] tiles handed out
+ * before their inputs were complete; [5] tiles taken from another XCD's queue. */
+int kleos_scheduler_stats(double stats[6]);
 
 /* ---- errors --------------------------------------------------------------------------------- */
 /* Replaces the KLEOS_CHECK_CUDA / KLEOS_ASSERT message conventions (csrc/include/kleos/debug.cuh:
