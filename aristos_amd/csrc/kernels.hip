@@ -234,18 +234,22 @@ __device__ __forceinline__ void expert_loop(const LayerParams& p, char* smem, ui
         G::begin(cur_t, args_of(cur), 0, smem);
         for (;;) {
             G::mainloop(cur_t, acc, smem);
-                Task nxt = next();   // its barrier: every wavefront has left the main loop
-                const bool early = nxt.valid && (nxt.kind == 0 || nxt.ready);
+            Task nxt = next();   // its barrier: every wavefront has left the main loop
+            const bool early = nxt.valid && (nxt.kind == 0 || nxt.ready);
             if (early) {
                 // the next tile's index look-ups and first loads travel while this tile's epilogue runs
                 acquire(nxt);
                 G::begin(nxt_t, args_of(nxt), G::next_stage0(cur_t), smem);
             }
-                G::finish(cur_t, acc, smem);
+            G::finish(cur_t, acc, smem);
+            if (rd.sched && cur.kind == 0) {
+                // an up-projection tile other workgroups wait for: its stores must be complete in
+                // every wavefront before it is counted
                 wait_vmcnt<0>();
-            __syncthreads();
-            publish(cur);
-                if (!nxt.valid) break;
+                __syncthreads();
+                publish(cur);
+            }
+            if (!nxt.valid) break;
             if (!early) {
                 wait_ready(nxt);
                 acquire(nxt);
