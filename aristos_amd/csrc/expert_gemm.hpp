@@ -31,7 +31,7 @@ namespace kleos_amd {
 // i.e. the core computes C^T: a lane then owns 4 consecutive output columns of one output row.
 //
 // The tile computation is split into the pieces a persistent workgroup overlaps across tiles:
-//   begin()    per-lane source addresses + the loads of the first STAGES-1 slices
+//   begin()    per-lane source addresses + the loads of the bias and of the first STAGES-1 slices
 //   mainloop() all K slices
 //   finish()   bias, activation, rounding, transposition through LDS, coalesced stores
 // A workgroup calls begin() of its next tile between mainloop() and finish() of the current one,
@@ -73,7 +73,9 @@ struct GemmBf16 {
     static constexpr int kChunks = kRowBytes / 16;                 // 16-byte chunks per row
     static constexpr int kABytes = BM * kRowBytes, kBBytes = BN * kRowBytes;
     static constexpr int kStage = kABytes + kBBytes;
-    static constexpr int kSmemBytes = STAGES * kStage;
+    static constexpr int kBiasBytes = BN * 2;                      // one tile's bias entries
+    static constexpr int kBiasOffset = STAGES * kStage;            // two bias slots behind the stage ring
+    static constexpr int kSmemBytes = STAGES * kStage + 2 * kBiasBytes;
     static constexpr int LA = BM / (kRowsPerLoad * kWaves), LB = BN / (kRowsPerLoad * kWaves);
     static constexpr int kLoadsPerSlice = LA + LB;                 // per wavefront
     static constexpr int kSteps = BK / 16;                         // matrix instructions consume 16 values of K
@@ -84,6 +86,7 @@ struct GemmBf16 {
     static_assert(BM % (kRowsPerLoad * kWaves) == 0 && BN % (kRowsPerLoad * kWaves) == 0);
     static_assert(kWaves * kPanelRows * 128 <= kStage, "epilogue staging must fit one stage");
     static_assert((STAGES - 1) * kLoadsPerSlice < 64);
+    static_assert(kBiasBytes <= 1024, "one direct load brings the bias");
 
     static __device__ __forceinline__ int swizzle(int r) {
         if constexpr (BK == 64) return ((r >> 1) & 7) ^ ((r & 1) << 2);
@@ -93,11 +96,20 @@ struct GemmBf16 {
     struct Tile {
         const bf16_t* pa[LA];
         const bf16_t* pb[LB];
-        const bf16_t* bias;
         bf16_t* c_base;
         uint32_t ldc, m_valid, n_valid, k_tiles, act;
         int stage0;                 // stage of K slice 0; slice kt uses (stage0 + kt) % STAGES
+        int bias_slot;              // which of the two LDS bias slots holds this tile's bias
     };
+
+    // The lane's thread index as a value the optimiser cannot trace back to threadIdx: whatever a
+    // phase derives from it is computed when the phase starts and dies when it ends, instead of
+    // being shared with the main loop and kept (or spilled) across it.
+    static __device__ __forceinline__ uint32_t local_tid() {
+        uint32_t t = threadIdx.x;
+        asm volatile("" : "+v"(t));
+        return t;
+    }
 
     typedef f32x16 Acc[TN][TM];
 
@@ -119,12 +131,19 @@ struct GemmBf16 {
                 __builtin_amdgcn_global_load_lds((global_cptr)(t.pb[i] + k0), (lds_ptr)(sb + 1024 * (wave + kWaves * i)), 16, 0, 0);
     }
 
-    // Per-lane source addresses, then the loads of the first STAGES-1 slices. Rows past the valid
-    // range re-read the last valid row: their products land in accumulator rows / columns that are
-    // never stored. The stages stage0 .. stage0+STAGES-2 must not be in use by any wavefront.
-    static __device__ __forceinline__ void begin(Tile& t, const GemmTileArgs& g, int stage0, char* smem) {
-        const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    // Per-lane source addresses, the load of the bias into LDS slot `bias_slot`, then the loads of
+    // the first STAGES-1 slices. Rows past the valid range re-read the last valid row: their
+    // products land in accumulator rows / columns that are never stored. The stages stage0 ..
+    // stage0+STAGES-2 and the bias slot must not be in use by any wavefront. The bias load is the
+    // oldest of the tile's loads, so the first wait of mainloop() covers it.
+    static __device__ __forceinline__ void begin(Tile& t, const GemmTileArgs& g, int stage0, int bias_slot, char* smem) {
+        const uint32_t tid = local_tid();
+        const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
         const int ld_r = lane / kChunks, ld_p = lane % kChunks;
+        if (wave == 0 && lane < kBiasBytes / 16) {
+            const uint32_t n = uint32_t(lane) * 8 < g.n_valid ? uint32_t(lane) * 8 : 0u;
+            __builtin_amdgcn_global_load_lds((global_cptr)(g.bias + n), (lds_ptr)(smem + kBiasOffset + bias_slot * kBiasBytes), 16, 0, 0);
+        }
 #pragma unroll
         for (int i = 0; i < LA; ++i) {
             const int row = kRowsPerLoad * (wave + kWaves * i) + ld_r;
@@ -138,9 +157,9 @@ struct GemmBf16 {
             const uint32_t r = row < int(g.n_valid) ? row : g.n_valid - 1;
             t.pb[i] = g.b_base + size_t(r) * g.ldb + ((ld_p ^ swizzle(row)) << 3);
         }
-        t.bias = g.bias; t.c_base = g.c_base; t.ldc = g.ldc;
+        t.c_base = g.c_base; t.ldc = g.ldc;
         t.m_valid = g.m_valid; t.n_valid = g.n_valid; t.k_tiles = g.K / BK;
-        t.act = g.act; t.stage0 = stage0;
+        t.act = g.act; t.stage0 = stage0; t.bias_slot = bias_slot;
 #pragma unroll
         for (int st = 0; st < STAGES - 1; ++st)
             if (uint32_t(st) < t.k_tiles) issue_part(t, smem, st, 0, 1);
@@ -199,17 +218,21 @@ struct GemmBf16 {
     static __device__ __forceinline__ int next_stage0(const Tile& t) { return (t.stage0 + t.k_tiles) % STAGES; }
 
     template <int ACT>
-    static __device__ __forceinline__ void finish_act(const Tile& t, Acc& acc, char* stage_mem) {
+    static __device__ __forceinline__ void finish_act(const Tile& t, Acc& acc, char* stage_mem, const char* bias_mem) {
         // acc[ni][mi][v] is output column n = wn*WN + ni*32 + 8*(v/4) + 4*(lane/32) + v%4 of output row
         // m = wm*WM + mi*32 + lane%32: a lane owns 4 consecutive columns of 16 rows per 32x32 block.
         // Bias, activation and the rounding to Element happen in registers; the wavefront then
         // transposes 32-row x 64-column panels through a private LDS region (rows of 128 bytes,
         // 16-byte chunk c of row r at position c ^ ((r >> 1) & 7)) so that the global stores are
-        // 16 bytes per lane and cover whole 128-byte lines of the output rows.
-        const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+        // 16 bytes per lane and cover whole 128-byte lines of the output rows. The bias comes from
+        // the tile's LDS slot: the epilogue issues no global load, so nothing in it ever waits for
+        // the stores it has in flight.
+        const uint32_t tid = local_tid();
+        const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
         const int wm = wave / WAVES_N, wn = wave % WAVES_N;
         const int fr_row = lane & 31, fr_half = lane >> 5;
         char* stg = stage_mem + wave * (kPanelRows * 128);
+        const char* bias_lane = bias_mem + (wn * WN + 4 * fr_half) * 2;
 #pragma unroll
         for (int mi = 0; mi < TM; ++mi) {
 #pragma unroll
@@ -219,16 +242,11 @@ struct GemmBf16 {
                     const int ni = pn * 2 + nl;
 #pragma unroll
                     for (int q = 0; q < 4; ++q) {
-                        const uint32_t n = wn * WN + ni * 32 + 8 * q + 4 * fr_half;
-                        float bv[4] = {0.f, 0.f, 0.f, 0.f};
-                        if (n < t.n_valid) {
-                            const bf16x4 b4 = *reinterpret_cast<const bf16x4*>(t.bias + n);
-#pragma unroll
-                            for (int j = 0; j < 4; ++j) bv[j] = float(b4[j]);
-                        }
+                        const bf16x4 b4 = *reinterpret_cast<const bf16x4*>(bias_lane + (ni * 32 + 8 * q) * 2);
                         bf16x4 o;
 #pragma unroll
-                        for (int j = 0; j < 4; ++j) o[j] = static_cast<bf16_t>(activate<ACT>(acc[ni][mi][4 * q + j] + bv[j]));
+                        for (int j = 0; j < 4; ++j)
+                            o[j] = static_cast<bf16_t>(activate<ACT>(acc[ni][mi][4 * q + j] + float(b4[j])));
                         *reinterpret_cast<bf16x4*>(stg + fr_row * 128 + (((nl * 4 + q) ^ ((fr_row >> 1) & 7)) << 4) + fr_half * 8) = o;
                     }
                 }
@@ -249,9 +267,10 @@ struct GemmBf16 {
     // Epilogue. Every wavefront must have left mainloop().
     static __device__ __forceinline__ void finish(const Tile& t, Acc& acc, char* smem) {
         char* stage_mem = smem + last_stage(t) * kStage;
-        if (t.act == 0) finish_act<0>(t, acc, stage_mem);
-        else if (t.act == 1) finish_act<1>(t, acc, stage_mem);
-        else finish_act<2>(t, acc, stage_mem);
+        const char* bias_mem = smem + kBiasOffset + t.bias_slot * kBiasBytes;
+        if (t.act == 0) finish_act<0>(t, acc, stage_mem, bias_mem);
+        else if (t.act == 1) finish_act<1>(t, acc, stage_mem, bias_mem);
+        else finish_act<2>(t, acc, stage_mem, bias_mem);
     }
 };
 

@@ -231,7 +231,8 @@ __device__ __forceinline__ void expert_loop(const LayerParams& p, char* smem, ui
         if (!cur.valid) { flush_stats(); return; }
         if (cur.kind == 1 && !cur.ready) wait_ready(cur);
         acquire(cur);
-        G::begin(cur_t, args_of(cur), 0, smem);
+        int bias_slot = 0;
+        G::begin(cur_t, args_of(cur), 0, bias_slot, smem);
         for (;;) {
             G::mainloop(cur_t, acc, smem);
             Task nxt = next();   // its barrier: every wavefront has left the main loop
@@ -239,7 +240,7 @@ __device__ __forceinline__ void expert_loop(const LayerParams& p, char* smem, ui
             if (early) {
                 // the next tile's index look-ups and first loads travel while this tile's epilogue runs
                 acquire(nxt);
-                G::begin(nxt_t, args_of(nxt), G::next_stage0(cur_t), smem);
+                G::begin(nxt_t, args_of(nxt), G::next_stage0(cur_t), bias_slot ^= 1, smem);
             }
             G::finish(cur_t, acc, smem);
             if (rd.sched && cur.kind == 0) {
@@ -253,7 +254,7 @@ __device__ __forceinline__ void expert_loop(const LayerParams& p, char* smem, ui
             if (!early) {
                 wait_ready(nxt);
                 acquire(nxt);
-                G::begin(nxt_t, args_of(nxt), G::next_stage0(cur_t), smem);
+                G::begin(nxt_t, args_of(nxt), G::next_stage0(cur_t), bias_slot ^= 1, smem);
             }
             cur = nxt;
             cur_t = nxt_t;

@@ -31,6 +31,12 @@ def main() -> int:
     ap.add_argument("--workload", default="headline_e64_zipf")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--calib-copy-mib", type=int, default=0,
+                    help="also run one device-to-device copy of this many MiB before the timed region "
+                         "(a kernel of known traffic to scale rocprofv3 FETCH_SIZE / WRITE_SIZE by)")
+    ap.add_argument("--traffic-bytes", type=float, default=None,
+                    help="measured HBM bytes per launch of the persistent kernel (from the rocprofv3 --pmc runs "
+                         "recorded under profiles/), reported as roofline.traffic")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures the single-GPU path (expert-parallel degree 1) only; run it with --gpus 1",
@@ -52,6 +58,14 @@ def main() -> int:
     torch.cuda.synchronize()
     bf16 = d.elem_bytes == 2
 
+    if args.calib_copy_mib > 0:
+        n = args.calib_copy_mib * (1 << 20)
+        src = torch.ones(n, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
     ka.initialize(w.config)
     try:
         oP = synth.alloc_outputs(d)
@@ -69,6 +83,8 @@ def main() -> int:
         wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
         # the same launches, timed by HIP events on the library stream (reference protocol, moe.cuh:160-181)
         ev_ms = ka.moe.forward_host_bench(iP, oP, skip=0, trials=args.steps)
+        fused_ph = ka.moe.phase_times()
+        sched = ka.moe.scheduler_stats()
         views = ka.moe.debug_views(d)
         kept = int(np.minimum(views["expert_count"].astype(np.int64), d.kept_capacity).sum())
         dropped = int((views["topk_slot"] < 0).sum())
@@ -86,7 +102,18 @@ def main() -> int:
     eb = d.elem_bytes
     peak = PEAK_BF16_TFLOPS if bf16 else PEAK_FP32_TFLOPS
     achieved = flops_layer / (ev_ms * 1e-3) / 1e12
+    # minimum HBM traffic of one forward: expert weights once + x (gate) + gathered rows + output + Wg
+    n_active = int((views["expert_count"] > 0).sum())
+    hbm_bytes = float(2 * n_active * d.H * d.I * eb + d.S * d.H * eb + kept * d.H * eb + d.S * d.H * eb + d.E * d.H * eb)
     up_dn_ms = ph["up"] + ph["down"]
+    ex_ms = fused_ph["up"]
+    fused_phases = {
+        "gate_ms": round(fused_ph["gate"], 4), "slots_ms": round(fused_ph["slots"], 4),
+        "experts_ms": round(ex_ms, 4), "combine_ms": round(fused_ph["combine"], 4),
+        "expert_gemm_tflops": round(flops_expert / (ex_ms * 1e-3) / 1e12, 2) if ex_ms > 0 else None,
+        "expert_gemm_mfma_frac": round(flops_expert / (ex_ms * 1e-3) / 1e12 / peak, 4) if ex_ms > 0 else None,
+        "scheduler": {k: round(v, 5) for k, v in sched.items()},
+    }
     phases = {
         "total_ms": round(ph_total, 4),
         "gate_ms": round(ph["gate"], 4), "slots_ms": round(ph["slots"], 4), "up_ms": round(ph["up"], 4),
@@ -122,10 +149,14 @@ def main() -> int:
         "tokens_per_s": round(d.S / (wall_ms * 1e-3), 1),
         "event_ms_per_step": round(ev_ms, 5),
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": peak, "unit": "TFLOP/s",
-                     "frac": round(achieved / peak, 4), "traffic": None,
+                     "frac": round(achieved / peak, 4), "traffic": args.traffic_bytes,
                      "kernel": "fused_kernel (whole layer: gate + slots + expert GEMMs + combine)",
-                     "flops_per_launch": flops_layer},
-        "phases": phases,
+                     "flops_per_launch": flops_layer,
+                     "hbm_algorithmic_bytes": hbm_bytes,
+                     "hbm_algorithmic_gbs": round(hbm_bytes / (ev_ms * 1e-3) / 1e9, 1),
+                     "hbm_peak_gbs": PEAK_HBM_GBS},
+        "fused_phases": fused_phases,
+        "phased_mode": phases,
         "cpu_baseline": cpu,
     }
     print(json.dumps(line))
