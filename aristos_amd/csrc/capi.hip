@@ -365,6 +365,21 @@ extern "C" int kleos_scheduler_stats(double stats[6]) {
     return KLEOS_OK;
 }
 
+extern "C" int kleos_phase_stamps(unsigned long long* stamps, uint32_t max_workgroups, uint32_t* n_workgroups) {
+    if (int rc = require_ctx("kleos_phase_stamps")) return rc;
+    if (!stamps || !n_workgroups) return fail(KLEOS_EINVAL, "kleos_phase_stamps: null argument");
+    Context& c = *g_ctx;
+    KLEOS_HIP(hipSetDevice(c.device));
+    KLEOS_HIP(hipStreamSynchronize(c.stream));
+    *n_workgroups = c.plan.nwg;
+    const uint32_t n = std::min(c.plan.nwg, max_workgroups);
+    std::vector<unsigned long long> st(size_t(n) * 16);
+    if (n) KLEOS_HIP(hipMemcpy(st.data(), c.base.stamps, st.size() * 8, hipMemcpyDeviceToHost));
+    for (uint32_t w = 0; w < n; ++w)
+        for (int i = 0; i < 8; ++i) stamps[size_t(w) * 8 + i] = st[size_t(w) * 16 + i];
+    return KLEOS_OK;
+}
+
 extern "C" int kleos_phase_times(float ms[5]) {
     if (int rc = require_ctx("kleos_phase_times")) return rc;
     if (!ms) return fail(KLEOS_EINVAL, "kleos_phase_times: null argument");

@@ -12,100 +12,147 @@
 
 namespace kleos_amd {
 
-// One token per wavefront; each lane handles 16-byte chunks of the row. The routing of the token
-// (at most kCombineInline experts on the fast path) is read once, then the expert rows of two
-// column chunks are requested together so that a wavefront keeps 2k loads in flight.
-constexpr int kCombineInline = 8;
+// One token per wavefront at a time; each lane handles 16-byte chunks of the row. A wavefront walks
+// the tokens first, first + stride, ... and keeps two things in flight while it sums a token: all
+// the expert rows of CH column chunks of that token, and the routing entries of its next token.
+// Everything it reads was written by other workgroups of the same launch (routing by the gate and
+// slot phases, y by the down-projection), hence the device-coherent loads; each y row is read
+// exactly once, so nothing is lost by not serving it from the L2.
+template <int KMAX>
+struct CombineRoute {
+    int32_t slot[KMAX];
+    int32_t expert[KMAX];
+    float prob[KMAX];
+    float den;
+};
 
-template <typename T>
-__device__ __forceinline__ void combine_token(const LayerParams& p, uint32_t token) {
+template <int KMAX>
+__device__ __forceinline__ CombineRoute<KMAX> combine_route(const LayerParams& p, uint32_t token) {
+    CombineRoute<KMAX> r;
+    r.den = load_coherent(p.combine_den + token);
+#pragma unroll
+    for (int i = 0; i < KMAX; ++i) {
+        r.slot[i] = -1; r.expert[i] = 0; r.prob[i] = 0.f;
+        if (uint32_t(i) < p.k) {
+            r.slot[i] = load_coherent(p.topk_slot + size_t(token) * p.k + i);
+            r.expert[i] = load_coherent(p.topk_expert + size_t(token) * p.k + i);
+            r.prob[i] = load_coherent(p.topk_prob + size_t(token) * p.k + i);
+        }
+    }
+    return r;
+}
+
+template <typename T, int KMAX, int CH>
+__device__ __forceinline__ void combine_tokens_inline(const LayerParams& p, uint32_t first, uint32_t stride) {
     constexpr int kPer = 16 / sizeof(T);
     const int lane = threadIdx.x & 63;
     const uint32_t H = p.H, k = p.k;
     const T* y = static_cast<const T*>(p.y);
-    T* out = static_cast<T*>(p.moe_out) + size_t(token) * H;
-    const float den = p.combine_den[token];
-    const uint32_t stride = kWave * kPer;
+    const uint32_t col_stride = kWave * kPer;
 
-    // Element(gateOut[t, e]) * Element(fp32(y) / den), summed in fp32 in selection order
-    // (processor.cuh:117,135,146); with k == 1 the row is copied unscaled (processor.cuh:170-203).
-    auto accumulate = [&](float (&accv)[kPer], const u32x4& raw, float scale) {
-        T vals[kPer];
-        __builtin_memcpy(vals, &raw, 16);
-        if (k == 1) {
+    if (first >= p.S) return;
+    CombineRoute<KMAX> cur = combine_route<KMAX>(p, first);
+    for (uint32_t token = first; token < p.S; token += stride) {
+        CombineRoute<KMAX> nxt = cur;
+        if (token + stride < p.S) nxt = combine_route<KMAX>(p, token + stride);
+        const float den = cur.den;
+        coherent_rows_t rows[KMAX];
+        float scale[KMAX];
+        bool on[KMAX];
 #pragma unroll
-            for (int j = 0; j < kPer; ++j) accv[j] = elem_to_float(vals[j]);
-        } else {
-#pragma unroll
-            for (int j = 0; j < kPer; ++j)
-                accv[j] = fmaf(scale, elem_to_float(float_to_elem<T>(elem_to_float(vals[j]) / den)), accv[j]);
+        for (int r = 0; r < KMAX; ++r) {
+            on[r] = cur.slot[r] >= 0;   // the same in every lane: a wavefront works on one token
+            // (indices clamped to their tables: no value they could hold leaves the y buffer)
+            const uint32_t e = uint32_t(cur.expert[r]) < p.E ? uint32_t(cur.expert[r]) : p.E - 1;
+            const uint32_t sl = uint32_t(cur.slot[r]) < p.cap_rows ? uint32_t(cur.slot[r]) : p.cap_rows - 1;
+            const size_t row = on[r] ? size_t(e) * p.cap_rows + sl : 0;
+            rows[r] = coherent_rows(y + row * H);
+            scale[r] = elem_to_float(float_to_elem<T>(cur.prob[r]));
         }
-    };
-    auto store_row = [&](uint32_t c0, const float (&accv)[kPer]) {
-        T o[kPer];
+        T* out = static_cast<T*>(p.moe_out) + size_t(token) * H;
+        for (uint32_t c0 = lane * kPer; c0 < H; c0 += CH * col_stride) {
+            u32x4 v[CH][KMAX];
 #pragma unroll
-        for (int j = 0; j < kPer; ++j) o[j] = float_to_elem<T>(accv[j]);
-        u32x4 raw;
-        __builtin_memcpy(&raw, o, 16);
-        store16(out + c0, raw);
-    };
-
-    if (k <= uint32_t(kCombineInline)) {
-        const T* row[kCombineInline];
-        float scale[kCombineInline];
+            for (int c = 0; c < CH; ++c)
 #pragma unroll
-        for (int r = 0; r < kCombineInline; ++r) {
-            row[r] = nullptr;
-            scale[r] = 0.f;
-            if (uint32_t(r) < k) {
-                const int32_t slot = p.topk_slot[size_t(token) * k + r];
-                if (slot >= 0) {
-                    const uint32_t e = uint32_t(p.topk_expert[size_t(token) * k + r]);
-                    row[r] = y + (size_t(e) * p.cap_rows + uint32_t(slot)) * H;
-                    scale[r] = elem_to_float(float_to_elem<T>(p.topk_prob[size_t(token) * k + r]));
+                for (int r = 0; r < KMAX; ++r)
+                    if (on[r] && c0 + c * col_stride < H) v[c][r] = load16_coherent(rows[r], (c0 + c * col_stride) * sizeof(T));
+#pragma unroll
+            for (int c = 0; c < CH; ++c) {
+                if (c0 + c * col_stride >= H) break;
+                // Element(gateOut[t, e]) * Element(fp32(y) / den), summed in fp32 in selection order
+                // (processor.cuh:117,135,146); with k == 1 the row is copied unscaled
+                // (processor.cuh:170-203).
+                float acc[kPer];
+#pragma unroll
+                for (int j = 0; j < kPer; ++j) acc[j] = 0.f;
+#pragma unroll
+                for (int r = 0; r < KMAX; ++r) {
+                    if (!on[r]) continue;
+                    T vals[kPer];
+                    __builtin_memcpy(vals, &v[c][r], 16);
+#pragma unroll
+                    for (int j = 0; j < kPer; ++j) {
+                        if (k == 1) acc[j] = elem_to_float(vals[j]);
+                        else acc[j] = fmaf(scale[r], elem_to_float(float_to_elem<T>(elem_to_float(vals[j]) / den)), acc[j]);
+                    }
                 }
+                T o[kPer];
+#pragma unroll
+                for (int j = 0; j < kPer; ++j) o[j] = float_to_elem<T>(acc[j]);
+                u32x4 raw;
+                __builtin_memcpy(&raw, o, 16);
+                store16(out + c0 + c * col_stride, raw);
             }
         }
-        uint32_t c0 = lane * kPer;
-        for (; c0 + stride < H; c0 += 2 * stride) {
-            u32x4 v0[kCombineInline], v1[kCombineInline];
-#pragma unroll
-            for (int r = 0; r < kCombineInline; ++r)
-                if (row[r]) { v0[r] = load16(row[r] + c0); v1[r] = load16(row[r] + c0 + stride); }
-            float a0[kPer], a1[kPer];
-#pragma unroll
-            for (int j = 0; j < kPer; ++j) { a0[j] = 0.f; a1[j] = 0.f; }
-#pragma unroll
-            for (int r = 0; r < kCombineInline; ++r)
-                if (row[r]) { accumulate(a0, v0[r], scale[r]); accumulate(a1, v1[r], scale[r]); }
-            store_row(c0, a0);
-            store_row(c0 + stride, a1);
-        }
-        for (; c0 < H; c0 += stride) {
-            float a0[kPer];
-#pragma unroll
-            for (int j = 0; j < kPer; ++j) a0[j] = 0.f;
-#pragma unroll
-            for (int r = 0; r < kCombineInline; ++r)
-                if (row[r]) accumulate(a0, load16(row[r] + c0), scale[r]);
-            store_row(c0, a0);
-        }
-        return;
+        cur = nxt;
     }
+}
 
-    for (uint32_t c0 = lane * kPer; c0 < H; c0 += stride) {
-        float accv[kPer];
+// Any k: the routing entries are re-read for every column chunk.
+template <typename T>
+__device__ __forceinline__ void combine_tokens_generic(const LayerParams& p, uint32_t first, uint32_t stride) {
+    constexpr int kPer = 16 / sizeof(T);
+    const int lane = threadIdx.x & 63;
+    const uint32_t H = p.H, k = p.k;
+    const T* y = static_cast<const T*>(p.y);
+    for (uint32_t token = first; token < p.S; token += stride) {
+        const float den = load_coherent(p.combine_den + token);
+        T* out = static_cast<T*>(p.moe_out) + size_t(token) * H;
+        for (uint32_t c0 = lane * kPer; c0 < H; c0 += kWave * kPer) {
+            float acc[kPer];
 #pragma unroll
-        for (int j = 0; j < kPer; ++j) accv[j] = 0.f;
-        for (uint32_t r = 0; r < k; ++r) {
-            const int32_t slot = p.topk_slot[size_t(token) * k + r];
-            if (slot < 0) continue;
-            const uint32_t e = uint32_t(p.topk_expert[size_t(token) * k + r]);
-            const T* yrow = y + (size_t(e) * p.cap_rows + uint32_t(slot)) * H + c0;
-            accumulate(accv, load16(yrow), elem_to_float(float_to_elem<T>(p.topk_prob[size_t(token) * k + r])));
+            for (int j = 0; j < kPer; ++j) acc[j] = 0.f;
+            for (uint32_t r = 0; r < k; ++r) {
+                const int32_t slot = load_coherent(p.topk_slot + size_t(token) * k + r);
+                if (slot < 0) continue;
+                uint32_t e = uint32_t(load_coherent(p.topk_expert + size_t(token) * k + r));
+                if (e >= p.E || uint32_t(slot) >= p.cap_rows) continue;
+                const float scale = elem_to_float(float_to_elem<T>(load_coherent(p.topk_prob + size_t(token) * k + r)));
+                const u32x4 raw = load16_coherent(coherent_rows(y + (size_t(e) * p.cap_rows + uint32_t(slot)) * H), c0 * sizeof(T));
+                T vals[kPer];
+                __builtin_memcpy(vals, &raw, 16);
+#pragma unroll
+                for (int j = 0; j < kPer; ++j)
+                    acc[j] = fmaf(scale, elem_to_float(float_to_elem<T>(elem_to_float(vals[j]) / den)), acc[j]);
+            }
+            T o[kPer];
+#pragma unroll
+            for (int j = 0; j < kPer; ++j) o[j] = float_to_elem<T>(acc[j]);
+            u32x4 raw;
+            __builtin_memcpy(&raw, o, 16);
+            store16(out + c0, raw);
         }
-        store_row(c0, accv);
     }
+}
+
+// Tokens first, first + stride, ... of the calling wavefront.
+template <typename T>
+__device__ __forceinline__ void combine_tokens(const LayerParams& p, uint32_t first, uint32_t stride) {
+    if (p.k <= 2) combine_tokens_inline<T, 2, 4>(p, first, stride);
+    else if (p.k <= 4) combine_tokens_inline<T, 4, 4>(p, first, stride);
+    else if (p.k <= 8) combine_tokens_inline<T, 8, 2>(p, first, stride);
+    else combine_tokens_generic<T>(p, first, stride);
 }
 
 }  // namespace kleos_amd

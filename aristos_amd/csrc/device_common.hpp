@@ -77,4 +77,32 @@ __device__ __forceinline__ void atomic_store_relaxed(uint32_t* p, uint32_t v) {
     __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// Device-coherent reads of data another workgroup of the same launch wrote (and made visible with
+// a device-scope release). The eight L2 caches of the device are not coherent with each other, and
+// a line read in an earlier phase or launch may still sit in this XCD's L2: these loads carry the
+// agent scope (sc1), which the caches do not serve from such a line. Reading the few tables that
+// cross workgroups this way replaces invalidating the whole L2 after every grid-wide barrier.
+template <typename V>
+__device__ __forceinline__ V load_coherent(const V* p) {
+    static_assert(sizeof(V) == 4 || sizeof(V) == 8);
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// 16-byte variant: buffer loads take the cache policy as an operand. `rows` describes memory that
+// starts at a wavefront-uniform address; `byte_offset` may differ per lane.
+typedef __amdgpu_buffer_rsrc_t coherent_rows_t;
+__device__ __forceinline__ coherent_rows_t coherent_rows(const void* uniform_base) {
+    const uint64_t a = reinterpret_cast<uint64_t>(uniform_base);
+    // readfirstlane returns a signed int: both halves go through uint32_t before they are widened,
+    // or a low half with its top bit set would smear ones over the high half
+    const uint32_t lo = uint32_t(__builtin_amdgcn_readfirstlane(int(uint32_t(a))));
+    const uint32_t hi = uint32_t(__builtin_amdgcn_readfirstlane(int(uint32_t(a >> 32))));
+    const uint64_t u = (uint64_t(hi) << 32) | uint64_t(lo);
+    // raw buffer: stride 0, 2 GiB window, 32-bit data format
+    return __builtin_amdgcn_make_buffer_rsrc(reinterpret_cast<void*>(u), 0, 0x7fffffff, 0x00020000);
+}
+__device__ __forceinline__ u32x4 load16_coherent(coherent_rows_t rows, uint32_t byte_offset) {
+    constexpr int kAgentScope = 16;   // sc1
+    return __builtin_amdgcn_raw_buffer_load_b128(rows, int(byte_offset), 0, kAgentScope);
+}
+
 }  // namespace kleos_amd

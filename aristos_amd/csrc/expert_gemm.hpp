@@ -54,6 +54,7 @@ __device__ __forceinline__ void wait_vmcnt() {
 struct GemmTileArgs {
     const bf16_t* a_base;          // A rows (gathered through a_row_index when it is not null)
     const int32_t* a_row_index;
+    uint32_t a_rows;               // rows behind a_base: gathered indices are clamped below it
     const bf16_t* b_base;          // first of the tile's weight rows
     const bf16_t* bias;            // first of the tile's bias entries
     bf16_t* c_base;                // output element (row 0, column 0) of the tile
@@ -80,8 +81,13 @@ struct GemmBf16 {
     static constexpr int kLoadsPerSlice = LA + LB;                 // per wavefront
     static constexpr int kSteps = BK / 16;                         // matrix instructions consume 16 values of K
     static constexpr int kPanelRows = 32;                          // epilogue staging: 32 rows x 64 columns per wavefront
+#ifdef KLEOS_ISSUE_STEPS
+    static constexpr int kIssueSteps = KLEOS_ISSUE_STEPS;
+#else
+    static constexpr int kIssueSteps = kSteps;                     // K steps over which the next slice's loads are issued
+#endif
     static_assert(BK == 32 || BK == 64);
-    static_assert(STAGES == 2 || STAGES == 3);
+    static_assert(STAGES >= 2 && STAGES <= 4);
     static_assert(WM % 32 == 0 && WN % 64 == 0);
     static_assert(BM % (kRowsPerLoad * kWaves) == 0 && BN % (kRowsPerLoad * kWaves) == 0);
     static_assert(kWaves * kPanelRows * 128 <= kStage, "epilogue staging must fit one stage");
@@ -148,8 +154,15 @@ struct GemmBf16 {
         for (int i = 0; i < LA; ++i) {
             const int row = kRowsPerLoad * (wave + kWaves * i) + ld_r;
             const uint32_t r = row < int(g.m_valid) ? row : g.m_valid - 1;
-            const size_t src = g.a_row_index ? size_t(g.a_row_index[r]) : size_t(r);
-            t.pa[i] = g.a_base + src * g.lda + ((ld_p ^ swizzle(row)) << 3);
+            // the slot->token table was written earlier in the same launch, possibly on another XCD
+            // (an index is clamped to the table it points into, so that no value it could ever
+            // hold turns into an address outside the caller's buffer)
+            uint32_t src = r;
+            if (g.a_row_index) {
+                src = uint32_t(load_coherent(g.a_row_index + r));
+                src = src < g.a_rows ? src : g.a_rows - 1;
+            }
+            t.pa[i] = g.a_base + size_t(src) * g.lda + ((ld_p ^ swizzle(row)) << 3);
         }
 #pragma unroll
         for (int i = 0; i < LB; ++i) {
@@ -183,8 +196,10 @@ struct GemmBf16 {
         const int base_w = kABytes + rw * kRowBytes + ((fr_half ^ swizzle(rw)) << 4);
         for (uint32_t kt = 0; kt < t.k_tiles; ++kt) {
             // This wavefront's loads of slice kt are complete once only those of the later slices
-            // already issued (STAGES-2 of them, none at the end of the tile) are outstanding.
-            if (STAGES == 3 && kt + 1 < t.k_tiles) wait_vmcnt<(STAGES - 2) * kLoadsPerSlice>();
+            // already issued (STAGES-2 of them, fewer at the end of the tile) are outstanding.
+            const uint32_t later = t.k_tiles - 1 - kt;
+            if (STAGES >= 4 && later >= 2) wait_vmcnt<(STAGES >= 4 ? 2 : 0) * kLoadsPerSlice>();
+            else if (STAGES >= 3 && later >= 1) wait_vmcnt<(STAGES >= 3 ? 1 : 0) * kLoadsPerSlice>();
             else wait_vmcnt<0>();
             // every wavefront's share of slice kt is in LDS, and everyone has finished with the stage
             // the next loads overwrite (slice kt-1, or the previous tile's epilogue staging)
@@ -194,20 +209,27 @@ struct GemmBf16 {
             const uint32_t ahead = kt + STAGES - 1;
             const bool more = ahead < t.k_tiles;
             const char* st = smem + stage_of(t, kt) * kStage;
+            // The operand fragments of K step ks+1 are read from LDS while the matrix core works
+            // on step ks.
+            bf16x8 fw[2][TN], fx[2][TM];
+            auto read_fragments = [&](int ks) {
+#pragma unroll
+                for (int ni = 0; ni < TN; ++ni) fw[ks & 1][ni] = __builtin_bit_cast(bf16x8, load16(st + (base_w ^ (ks << 5)) + ni * 32 * kRowBytes));
+#pragma unroll
+                for (int mi = 0; mi < TM; ++mi) fx[ks & 1][mi] = __builtin_bit_cast(bf16x8, load16(st + (base_x ^ (ks << 5)) + mi * 32 * kRowBytes));
+            };
+            read_fragments(0);
 #pragma unroll
             for (int ks = 0; ks < kSteps; ++ks) {
-                bf16x8 fw[TN], fx[TM];
-#pragma unroll
-                for (int ni = 0; ni < TN; ++ni) fw[ni] = __builtin_bit_cast(bf16x8, load16(st + (base_w ^ (ks << 5)) + ni * 32 * kRowBytes));
-#pragma unroll
-                for (int mi = 0; mi < TM; ++mi) fx[mi] = __builtin_bit_cast(bf16x8, load16(st + (base_x ^ (ks << 5)) + mi * 32 * kRowBytes));
-                if (more) issue_part(t, smem, ahead, ks, kSteps);
+                if (ks + 1 < kSteps) read_fragments(ks + 1);
+                if (more && ks < kIssueSteps) issue_part(t, smem, ahead, ks, kIssueSteps);
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int ni = 0; ni < TN; ++ni)
 #pragma unroll
                     for (int mi = 0; mi < TM; ++mi)
-                        acc[ni][mi] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fw[ni], fx[mi], acc[ni][mi], 0, 0, 0);
+                        acc[ni][mi] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fw[ks & 1][ni], fx[ks & 1][mi], acc[ni][mi], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
     }
@@ -283,7 +305,7 @@ constexpr int gemm_f32_smem_bytes() { return 2 * kF32BK * kF32Pad * 4; }
 
 template <int ACT>
 __device__ __forceinline__ void gemm_tile_f32(
-    const float* __restrict__ a_base, const int32_t* __restrict__ a_row_index, uint32_t lda,
+    const float* __restrict__ a_base, const int32_t* __restrict__ a_row_index, uint32_t a_rows, uint32_t lda,
     uint32_t m_valid,
     const float* __restrict__ b_base, uint32_t ldb, uint32_t n_valid,
     const float* __restrict__ bias, float* __restrict__ c_base, uint32_t ldc, uint32_t K,
@@ -297,8 +319,13 @@ __device__ __forceinline__ void gemm_tile_f32(
     const float* pa = nullptr;
     const float* pb = nullptr;
     if (uint32_t(ld_row) < m_valid) {
-        const size_t src = a_row_index ? size_t(a_row_index[ld_row]) : size_t(ld_row);
-        pa = a_base + src * lda + ld_kq * 4;
+        // written earlier in the same launch, possibly on another XCD
+        uint32_t src = ld_row;
+        if (a_row_index) {
+            src = uint32_t(load_coherent(a_row_index + ld_row));
+            src = src < a_rows ? src : a_rows - 1;
+        }
+        pa = a_base + size_t(src) * lda + ld_kq * 4;
     }
     if (uint32_t(ld_row) < n_valid) pb = b_base + size_t(ld_row) * ldb + ld_kq * 4;
 

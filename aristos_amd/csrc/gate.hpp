@@ -224,7 +224,8 @@ __device__ __forceinline__ void gate_tile(const LayerParams& p, uint32_t tile, b
 
 // Slot assignment for one 16-token tile per wavefront. Every thread of the workgroup must call it
 // (it contains workgroup barriers); a wave without work passes valid = false. `base` is LDS
-// scratch of E uint32 private to the calling wave. Must run after every gate tile has finished.
+// scratch of E uint32 private to the calling wave. Must run after every gate tile has finished
+// and released its results; what the gate tiles wrote is read with device-coherent loads.
 //   slot = (tokens routed to e in all earlier tiles) + (rank inside this tile); a token keeps its
 //   expert iff slot < EC (gate.cuh:710-716).
 __device__ __forceinline__ void slot_tile(const LayerParams& p, uint32_t tile, bool valid,
@@ -232,30 +233,64 @@ __device__ __forceinline__ void slot_tile(const LayerParams& p, uint32_t tile, b
     const int lane = threadIdx.x & 63;
     const uint32_t E = p.E;
     const uint32_t* super = p.super_count + size_t(p.epoch & 1u) * p.n_super * E;
+    // The tile's (token, expert) pairs are requested first: they do not depend on the counts, and
+    // every dependent round trip to memory written by other XCDs costs more than a microsecond.
+    const uint32_t pairs = kGateTileTokens * p.k;
+    constexpr uint32_t kInline = 4;            // pairs per lane kept in registers (k <= 16)
+    uint32_t pe[kInline];
+    int32_t pr[kInline];
+#pragma unroll
+    for (uint32_t u = 0; u < kInline; ++u) {
+        const uint32_t i = lane + u * kWave;
+        pe[u] = 0; pr[u] = 0;
+        if (valid && i < pairs) {
+            pe[u] = uint32_t(load_coherent(p.topk_expert + size_t(tile) * pairs + i));
+            pr[u] = load_coherent(p.topk_slot + size_t(tile) * pairs + i);
+        }
+    }
     if (valid) {
         const uint32_t sup = tile / kSuperTiles;
+        const uint32_t first = sup * kSuperTiles;
+        // The coarse rows before this tile's block and the tile rows inside it form one list of
+        // n rows, summed per expert in batches of 16 loads that are in flight together (the row
+        // index is clamped instead of branching, so the loads of a batch issue back to back).
+        const uint32_t n = sup + (tile - first);
+        auto row_ptr = [&](uint32_t r) {
+            return r < sup ? super + size_t(r) * E : p.tile_count + size_t(first + (r - sup)) * E;
+        };
         for (uint32_t e = lane; e < E; e += kWave) {
             uint32_t acc = 0;
-            for (uint32_t s = 0; s < sup; ++s) acc += super[size_t(s) * E + e];
-            for (uint32_t j = sup * kSuperTiles; j < tile; ++j) acc += p.tile_count[size_t(j) * E + e];
+            constexpr uint32_t kBatch = 16;
+            for (uint32_t r0 = 0; r0 < n; r0 += kBatch) {
+                uint32_t v[kBatch];
+#pragma unroll
+                for (uint32_t u = 0; u < kBatch; ++u) v[u] = load_coherent(row_ptr(r0 + u < n ? r0 + u : n - 1) + e);
+#pragma unroll
+                for (uint32_t u = 0; u < kBatch; ++u) acc += r0 + u < n ? v[u] : 0u;
+            }
             base[e] = acc;
             // total routed per expert, dropped tokens included (the reference's eC, gate.cuh:699)
             if (tile + 1 == p.n_gate_tiles)
-                p.expert_count[e] = acc + p.tile_count[size_t(tile) * E + e];
+                p.expert_count[e] = acc + load_coherent(p.tile_count + size_t(tile) * E + e);
         }
     }
     __syncthreads();
     if (valid) {
-        const uint32_t pairs = kGateTileTokens * p.k;
-        for (uint32_t i = lane; i < pairs; i += kWave) {
+        auto assign = [&](uint32_t i, uint32_t e, int32_t rank) {
             const size_t idx = size_t(tile) * pairs + i;
             const uint32_t token = tile * kGateTileTokens + i / p.k;
-            const uint32_t e = uint32_t(p.topk_expert[idx]);
-            const uint32_t slot = base[e] + uint32_t(p.topk_slot[idx]);
+            if (e >= E) e = E - 1;   // cannot happen; keeps every address below inside its table
+            const uint32_t slot = base[e] + uint32_t(rank);
             const bool keep = slot < p.EC && slot < p.cap_rows;
             p.topk_slot[idx] = keep ? int32_t(slot) : -1;
             if (keep) p.slot_token[size_t(e) * p.cap_rows + slot] = int32_t(token);
-        }
+        };
+#pragma unroll
+        for (uint32_t u = 0; u < kInline; ++u)
+            if (lane + u * kWave < pairs) assign(lane + u * kWave, pe[u], pr[u]);
+        for (uint32_t i = lane + kInline * kWave; i < pairs; i += kWave)
+            assign(i, uint32_t(load_coherent(p.topk_expert + size_t(tile) * pairs + i)),
+                   load_coherent(p.topk_slot + size_t(tile) * pairs + i));
     }
     __syncthreads();
 }

@@ -29,7 +29,10 @@ constexpr int kXcds = 8;
 // Expert GEMM configuration of the bf16 path: 256 x 256 tile (an expert's whole capacity of 256 rows
 // at the headline shape, so its weights stream from HBM exactly once), 2 x 4 wavefronts of 128 x 64
 // (two per SIMD), K slices of 64 (whole 128-byte lines of every row) through two 64 KB stages.
-using GemmCfg = GemmBf16<256, 256, 2, 4, 64, 2>;
+#ifndef KLEOS_GEMM_CFG
+#define KLEOS_GEMM_CFG 256, 256, 2, 4, 64, 2
+#endif
+using GemmCfg = GemmBf16<KLEOS_GEMM_CFG>;
 constexpr int kBM = 256, kBN = 256;
 constexpr int kGemmThreads = GemmCfg::kThreads;
 
@@ -50,25 +53,31 @@ constexpr int kStampWords = 16;         // per-workgroup phase stamps [0..7] and
 
 __host__ __device__ inline uint32_t ceil_div_u32(uint32_t a, uint32_t b) { return (a + b - 1) / b; }
 
+// kCoherent: the counts were written earlier in the same launch (persistent kernel).
+template <bool kCoherent>
 __device__ __forceinline__ uint32_t kept_rows(const LayerParams& p, uint32_t e) {
     // consumers clamp the routed count to the capacity (packet.cuh:85,112-113)
-    const uint32_t c = p.expert_count[e];
+    const uint32_t c = kCoherent ? load_coherent(p.expert_count + e) : p.expert_count[e];
     const uint32_t cap = p.EC < p.cap_rows ? p.EC : p.cap_rows;
     return c < cap ? c : cap;
 }
 
 // ------------------------------------------------------------------------------------ scheduler state
-// Scheduler words (uint32), all in p.sched:
-//   [0..2]                 grid-barrier arrival counters, monotonically increasing across launches
-//   [8..15]                ticket counter of each XCD queue
-//   [16 .. 16+E*mt_max)    readiness: up-projection tiles stored per (expert, row block)
-//   [4]                    set to non-zero by a workgroup whose bounded wait expired
-constexpr uint32_t kSchedBar = 0, kSchedError = 4, kSchedTicket = 8, kSchedReady = 16;
+// Scheduler words (uint32), all in p.sched. Counters that different workgroups hit at the same
+// time sit on 128-byte lines of their own (kSchedLine words apart): atomics on one line serialise.
+//   kSchedBar + 32 b              grid barrier b: groups that have arrived, monotonic across launches
+//   kSchedGroup + 32 (8 b + g)    grid barrier b: arrivals of workgroup group g, monotonic
+//   kSchedTicket + 32 q           ticket counter of XCD queue q
+//   kSchedReady + e*mt_max + m    readiness: up-projection tiles stored per (expert, row block)
+//   kSchedError                   set to non-zero by a workgroup whose bounded wait expired
+constexpr uint32_t kSchedLine = 32;
+constexpr uint32_t kSchedBar = 0, kSchedError = 4, kSchedTicket = 4 * kSchedLine, kSchedGroup = 12 * kSchedLine,
+                   kSchedReady = 36 * kSchedLine;
 // Every wait in the persistent kernel is bounded so that the grid always drains: after this many
 // ticks of the 100 MHz wall clock a waiter records an error and proceeds.
 constexpr unsigned long long kWaitTicks = 300000000ull;   // 3 s
 // LDS header of the expert phase (bytes)
-constexpr size_t kLdsMt = 512, kLdsQueue = 128, kLdsSeg = 8 * (2 * 16 * kMaxGateGroups);
+constexpr size_t kLdsMt = 1536, kLdsQueue = 256, kLdsSeg = 8 * (2 * 16 * kMaxGateGroups);
 constexpr size_t kFusedLdsHeader = kLdsMt + kLdsQueue + kLdsSeg;
 
 struct Segment {
@@ -92,16 +101,33 @@ __device__ __forceinline__ void bounded_wait(uint32_t* sched, Pred&& pred) {
     }
 }
 
-__device__ __forceinline__ void grid_barrier(uint32_t* sched, uint32_t which, uint32_t target) {
-    uint32_t* ctr = sched + kSchedBar + which;
+// Grid-wide barrier number `which` of persistent launch number `seq` (launches counted from 0 on
+// this arena) of a grid of `nwg` resident workgroups. Arrivals are counted in two levels, eight
+// groups of workgroups (id mod 8) whose last member reports the group: a few dozen atomics land on
+// each counter instead of one per workgroup on a single word, which is what a flat barrier spends
+// most of its time on when everybody arrives together. All counters only ever grow, so nothing is
+// reset between launches.
+__device__ __forceinline__ void grid_barrier(uint32_t* sched, uint32_t which, uint32_t seq, uint32_t nwg) {
     __syncthreads();
     if (threadIdx.x == 0) {
+        const uint32_t g = blockIdx.x % kXcds;
+        const uint32_t members = (nwg - g + kXcds - 1) / kXcds;
+        const uint32_t groups = nwg < uint32_t(kXcds) ? nwg : uint32_t(kXcds);
+        uint32_t* all = sched + kSchedBar + which * kSchedLine;
+        uint32_t* mine = sched + kSchedGroup + (which * kXcds + g) * kSchedLine;
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-        atomic_add_agent(ctr, 1u);
-        bounded_wait(sched, [&] { return int32_t(atomic_load_relaxed(ctr) - target) >= 0; });
+        if (atomic_add_agent(mine, 1u) + 1u == (seq + 1u) * members) {
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "agent");
+            atomic_add_agent(all, 1u);
+        }
+        const uint32_t target = (seq + 1u) * groups;
+        bounded_wait(sched, [&] { return int32_t(atomic_load_relaxed(all) - target) >= 0; });
     }
     __syncthreads();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    // No device-scope acquire here: it would invalidate the whole L2 of the XCD (tens of
+    // microseconds of refetching per launch). What crosses workgroups after a barrier is read
+    // with device-coherent loads instead; this only drops the CU's own L1.
+    asm volatile("buffer_inv sc0" ::: "memory");
 }
 
 // One unit of expert work: an output tile of the up-projection (kind 0: h1 = act(x_gathered *
@@ -109,23 +135,27 @@ __device__ __forceinline__ void grid_barrier(uint32_t* sched, uint32_t which, ui
 // types.cuh:461). The reference's 128-byte Task descriptor (types.cuh:565-654) shrinks to this.
 struct Task {
     uint32_t e, kind, mtile, ntile;
+    uint32_t rows;      // rows the expert keeps (routed count clamped to the capacity)
     uint32_t foreign;   // taken from another XCD's queue: its h1 rows may sit in a different L2
+    uint32_t dep;       // down tile: the readiness counter of its row block as seen when handed out
     uint32_t ready;     // down tile whose up-projection row block was already complete when handed out
     uint32_t valid;
 };
-constexpr int kTaskWords = 8;
+constexpr int kTaskWords = 12;
 
 // Thread 0 publishes a task through LDS; every thread of the workgroup returns the same task.
 // The barrier inside also separates the caller's previous and next use of the LDS.
 __device__ __forceinline__ Task broadcast_task(uint32_t* s_task, const Task& mine) {
     if (threadIdx.x == 0) {
         s_task[0] = mine.e; s_task[1] = mine.kind; s_task[2] = mine.mtile; s_task[3] = mine.ntile;
-        s_task[4] = mine.foreign; s_task[5] = mine.ready; s_task[6] = mine.valid;
+        s_task[4] = mine.foreign; s_task[5] = mine.ready; s_task[6] = mine.valid; s_task[7] = mine.rows;
+        s_task[8] = mine.dep;
     }
     __syncthreads();
     Task t;
     t.e = s_task[0]; t.kind = s_task[1]; t.mtile = s_task[2]; t.ntile = s_task[3];
-    t.foreign = s_task[4]; t.ready = s_task[5]; t.valid = s_task[6];
+    t.foreign = s_task[4]; t.ready = s_task[5]; t.valid = s_task[6]; t.rows = s_task[7];
+    t.dep = s_task[8];
     return t;
 }
 
@@ -139,7 +169,7 @@ template <typename T>
 __device__ __forceinline__ TileOperands<T> tile_operands(const LayerParams& p, const Task& t) {
     constexpr int BM = TileShape<T>::BM, BN = TileShape<T>::BN;
     TileOperands<T> o;
-    const uint32_t rows = kept_rows(p, t.e);
+    const uint32_t rows = t.rows;
     const uint32_t row0 = t.mtile * BM, col0 = t.ntile * BN;
     const uint32_t N = t.kind == 0 ? p.I : p.H;
     o.K = t.kind == 0 ? p.H : p.I;
@@ -163,6 +193,11 @@ struct Readiness {
     uint32_t* sched;      // nullptr: no cross-tile dependencies inside this launch (phased mode)
     uint32_t mt_max, tn_up;
     __device__ __forceinline__ uint32_t* counter(const Task& t) const { return sched + kSchedReady + t.e * mt_max + t.mtile; }
+    // A counter holds the stored tiles of the row block in its low half and, in its high half, how
+    // many of them were stored by a workgroup on a foreign XCD (from whose L2 they were written back
+    // to memory, while this XCD's L2 may still hold the rows as an earlier launch left them).
+    static constexpr uint32_t kForeignUnit = 0x10000u;
+    __device__ __forceinline__ bool complete(uint32_t v) const { return (v & 0xffffu) >= tn_up; }
 };
 
 // The expert phase of one workgroup: tiles from `next` until it runs dry. `next()` is called by
@@ -184,11 +219,16 @@ __device__ __forceinline__ void expert_loop(const LayerParams& p, char* smem, ui
         if (t.valid) { ++n_tiles; n_late += !t.ready; n_foreign += t.foreign; }
         return t;
     };
-    auto wait_ready = [&](const Task& t) {
+    auto wait_ready = [&](Task& t) {
         // only a down tile handed out before its inputs were complete gets here
         const unsigned long long t0 = wall_clock64();
-        if (tid == 0) bounded_wait(rd.sched, [&] { return atomic_load_relaxed(rd.counter(t)) >= rd.tn_up; });
+        if (tid == 0) {
+            uint32_t seen = t.dep;
+            bounded_wait(rd.sched, [&] { seen = atomic_load_relaxed(rd.counter(t)); return rd.complete(seen); });
+            s_task[kTaskWords - 1] = seen;
+        }
         __syncthreads();
+        t.dep = s_task[kTaskWords - 1];
         st_wait += wall_clock64() - t0;
     };
     auto flush_stats = [&]() {
@@ -200,8 +240,9 @@ __device__ __forceinline__ void expert_loop(const LayerParams& p, char* smem, ui
         // Before a down tile reads h1 rows that other workgroups of this launch wrote: rows written
         // on this XCD are current in its L2, so dropping this CU's L1 is enough; rows written on
         // another XCD need the device-scope acquire, which also drops this XCD's stale L2 lines.
+        // The same holds for rows a foreign workgroup stored on behalf of this XCD's queue.
         if (!rd.sched || t.kind != 1) return;
-        if (t.foreign) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        if (t.foreign || t.dep >= Readiness::kForeignUnit) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
         else asm volatile("buffer_inv sc0" ::: "memory");
     };
     auto publish = [&](const Task& t) {
@@ -210,7 +251,7 @@ __device__ __forceinline__ void expert_loop(const LayerParams& p, char* smem, ui
         if (rd.sched && t.kind == 0 && tid == 0) {
             const unsigned long long t0 = wall_clock64();
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-            atomic_add_agent(rd.counter(t), 1u);
+            atomic_add_agent(rd.counter(t), t.foreign ? 1u + Readiness::kForeignUnit : 1u);
             st_pub += wall_clock64() - t0;
         }
     };
@@ -220,7 +261,7 @@ __device__ __forceinline__ void expert_loop(const LayerParams& p, char* smem, ui
         auto args_of = [&](const Task& t) {
             const TileOperands<T> o = tile_operands<T>(p, t);
             GemmTileArgs g;
-            g.a_base = o.a; g.a_row_index = o.idx; g.b_base = o.w; g.bias = o.bias; g.c_base = o.c;
+            g.a_base = o.a; g.a_row_index = o.idx; g.a_rows = p.S; g.b_base = o.w; g.bias = o.bias; g.c_base = o.c;
             g.lda = o.lda; g.ldb = o.K; g.ldc = o.ldc; g.K = o.K; g.m_valid = o.m_valid; g.n_valid = o.n_valid;
             g.act = o.act;
             return g;
@@ -262,14 +303,14 @@ __device__ __forceinline__ void expert_loop(const LayerParams& p, char* smem, ui
         flush_stats();
     } else {
         for (;;) {
-            const Task t = next();
+            Task t = next();
             if (!t.valid) break;
             if (t.kind == 1 && !t.ready) wait_ready(t);
             acquire(t);
             const TileOperands<T> o = tile_operands<T>(p, t);
-            if (o.act == 0) gemm_tile_f32<0>(o.a, o.idx, o.lda, o.m_valid, o.w, o.K, o.n_valid, o.bias, o.c, o.ldc, o.K, smem);
-            else if (o.act == 1) gemm_tile_f32<1>(o.a, o.idx, o.lda, o.m_valid, o.w, o.K, o.n_valid, o.bias, o.c, o.ldc, o.K, smem);
-            else gemm_tile_f32<2>(o.a, o.idx, o.lda, o.m_valid, o.w, o.K, o.n_valid, o.bias, o.c, o.ldc, o.K, smem);
+            if (o.act == 0) gemm_tile_f32<0>(o.a, o.idx, p.S, o.lda, o.m_valid, o.w, o.K, o.n_valid, o.bias, o.c, o.ldc, o.K, smem);
+            else if (o.act == 1) gemm_tile_f32<1>(o.a, o.idx, p.S, o.lda, o.m_valid, o.w, o.K, o.n_valid, o.bias, o.c, o.ldc, o.K, smem);
+            else gemm_tile_f32<2>(o.a, o.idx, p.S, o.lda, o.m_valid, o.w, o.K, o.n_valid, o.bias, o.c, o.ldc, o.K, smem);
             __syncthreads();
             publish(t);
         }
@@ -321,8 +362,9 @@ __global__ __launch_bounds__(TileShape<T>::kThreads, TileShape<T>::kPerCu) void 
                     rem = i % per_expert;
                 }
                 const uint32_t mtile = rem % tiles_m;
-                if (mtile * TileShape<T>::BM >= kept_rows(p, e)) continue;   // the expert has fewer rows
-                t.e = e; t.kind = kind; t.mtile = mtile; t.ntile = rem / tiles_m; t.ready = 1; t.valid = 1;
+                const uint32_t rows = kept_rows<false>(p, e);
+                if (mtile * TileShape<T>::BM >= rows) continue;   // the expert has fewer rows
+                t.e = e; t.rows = rows; t.kind = kind; t.mtile = mtile; t.ntile = rem / tiles_m; t.ready = 1; t.valid = 1;
                 i += gridDim.x;
                 break;
             }
@@ -335,12 +377,12 @@ __global__ __launch_bounds__(TileShape<T>::kThreads, TileShape<T>::kPerCu) void 
 template <typename T>
 __global__ __launch_bounds__(kPhaseThreads) void combine_kernel(const LayerParams p) {
     const uint32_t token = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (token < p.S) combine_token<T>(p, token);
+    combine_tokens<T>(p, token, p.S);
 }
 
 // ------------------------------------------------------------------------------------ fused
 template <typename T, int NG>
-__global__ __launch_bounds__(TileShape<T>::kThreads, TileShape<T>::kPerCu) void fused_kernel(const LayerParams p, uint32_t barrier_base,
+__global__ __launch_bounds__(TileShape<T>::kThreads, TileShape<T>::kPerCu) void fused_kernel(const LayerParams p, uint32_t seq,
                                                                       uint32_t mt_max, uint32_t lag) {
     static_assert(sizeof(Segment) == 8, "segment table sizing");
     extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -356,30 +398,33 @@ __global__ __launch_bounds__(TileShape<T>::kThreads, TileShape<T>::kPerCu) void 
     // ---- phase 0: gate. Workgroup 0 also resets this launch's tickets and readiness counters;
     // nothing reads them before the second barrier.
     if (blockIdx.x == 0) {
-        for (uint32_t i = tid; i < kXcds + p.E * mt_max; i += kThreads) sched[kSchedTicket + i] = 0u;
+        if (tid < uint32_t(kXcds)) sched[kSchedTicket + tid * kSchedLine] = 0u;
+        for (uint32_t i = tid; i < p.E * mt_max; i += kThreads) sched[kSchedReady + i] = 0u;
     }
     for (uint32_t t0 = blockIdx.x * kGroups; t0 < p.n_gate_tiles; t0 += nwg * kGroups)
         gate_tile<T, NG>(p, t0 + group, t0 + group < p.n_gate_tiles,
                          reinterpret_cast<float*>(smem) + group * gate_smem_floats<NG>());
     if (tid == 0) stamp[1] = wall_clock64();
-    grid_barrier(sched, 0, barrier_base + nwg);
+    grid_barrier(sched, 0, seq, nwg);
     if (tid == 0) stamp[2] = wall_clock64();
 
     // ---- phase 1: slots in token order
     {
         uint32_t* base = reinterpret_cast<uint32_t*>(smem) + wave * p.E;
-        for (uint32_t t0 = blockIdx.x * kWaves; t0 < p.n_gate_tiles; t0 += nwg * kWaves)
-            slot_tile(p, t0 + wave, t0 + wave < p.n_gate_tiles, base);
+        // wavefront w of workgroup b takes tile b + w * nwg: the tiles spread over all CUs
+        for (uint32_t t0 = blockIdx.x; t0 < p.n_gate_tiles; t0 += nwg * kWaves)
+            slot_tile(p, t0 + wave * nwg, t0 + wave * nwg < p.n_gate_tiles, base);
         uint32_t* other = p.super_count + size_t((p.epoch & 1u) ^ 1u) * p.n_super * p.E;
         for (uint32_t i = blockIdx.x * kThreads + tid; i < p.n_super * p.E; i += nwg * kThreads) other[i] = 0u;
     }
     if (tid == 0) stamp[3] = wall_clock64();
-    grid_barrier(sched, 1, barrier_base + nwg);
+    grid_barrier(sched, 1, seq, nwg);
     if (tid == 0) stamp[4] = wall_clock64();
 
     // ---- phase 2: expert tiles from per-XCD ticket queues
     // LDS map: row blocks per expert | queue starts, totals, task | segments | GEMM tile
-    uint16_t* s_mt = reinterpret_cast<uint16_t*>(smem);                         // [E], E <= 256
+    uint32_t* s_rows = reinterpret_cast<uint32_t*>(smem);                       // [E], E <= 256: rows kept
+    uint16_t* s_mt = reinterpret_cast<uint16_t*>(smem + 1024);                  // [E] row blocks
     uint32_t* s_qseg = reinterpret_cast<uint32_t*>(smem + kLdsMt);              // [9] first segment of each queue
     uint32_t* s_qtot = s_qseg + 16;                                             // [8] tickets in each queue
     uint32_t* s_task = s_qtot + 8;                                              // [kTaskWords] task broadcast slot
@@ -387,7 +432,11 @@ __global__ __launch_bounds__(TileShape<T>::kThreads, TileShape<T>::kPerCu) void 
     char* s_gemm = smem + kFusedLdsHeader;
     const uint32_t tn_up = ceil_div_u32(p.I, BN), tn_down = ceil_div_u32(p.H, BN);
 
-    for (uint32_t e = tid; e < p.E; e += kThreads) s_mt[e] = uint16_t(ceil_div_u32(kept_rows(p, e), BM));
+    for (uint32_t e = tid; e < p.E; e += kThreads) {
+        const uint32_t rows = kept_rows<true>(p, e);
+        s_rows[e] = rows;
+        s_mt[e] = uint16_t(ceil_div_u32(rows, BM));
+    }
     __syncthreads();
     if (tid == 0) {
         uint32_t nseg = 0;
@@ -421,15 +470,25 @@ __global__ __launch_bounds__(TileShape<T>::kThreads, TileShape<T>::kPerCu) void 
     // up-projection to its down-projection all live in one L2.
     const uint32_t xcd = __builtin_amdgcn_s_getreg((3 << 11) | 20) & (kXcds - 1);
     uint32_t q_off = 0;   // queues already found empty, starting from this workgroup's own XCD
+    uint32_t q_dead = 0;  // bit q: queue q was seen exhausted
+    bool q_scanned = false;
     const Readiness rd{sched, mt_max, tn_up};
     auto next = [&]() {
         Task t{};
         if (tid == 0) {
             while (q_off < kXcds) {
                 const uint32_t q = (xcd + q_off) % kXcds;
-                // cheap pre-check keeps exhausted queues from being hammered
-                if (s_qtot[q] == 0) { ++q_off; continue; }
-                const uint32_t ticket = atomic_add_agent(sched + kSchedTicket + q, 1u);
+                if (q_off != 0 && !q_scanned) {
+                    // Leaving the own queue: read every ticket counter once, all loads in flight
+                    // together, so that exhausted foreign queues (the normal case when the load is
+                    // balanced) cost one round trip in total instead of one atomic each.
+                    uint32_t seen[kXcds];
+                    for (uint32_t j = 0; j < kXcds; ++j) seen[j] = atomic_load_relaxed(sched + kSchedTicket + j * kSchedLine);
+                    for (uint32_t j = 0; j < kXcds; ++j) q_dead |= uint32_t(seen[j] >= s_qtot[j]) << j;
+                    q_scanned = true;
+                }
+                if (s_qtot[q] == 0 || ((q_dead >> q) & 1u)) { ++q_off; continue; }
+                const uint32_t ticket = atomic_add_agent(sched + kSchedTicket + q * kSchedLine, 1u);
                 if (ticket >= s_qtot[q]) { ++q_off; continue; }
                 uint32_t sg = s_qseg[q];
                 const uint32_t sg_end = s_qseg[q + 1];
@@ -439,8 +498,10 @@ __global__ __launch_bounds__(TileShape<T>::kThreads, TileShape<T>::kPerCu) void 
                 const uint32_t local = ticket - s_seg[sg].start;
                 t.mtile = local % s_mt[t.e];
                 t.ntile = local / s_mt[t.e];
+                t.rows = s_rows[t.e];
                 t.foreign = q_off != 0;
-                t.ready = t.kind == 0 || atomic_load_relaxed(rd.counter(t)) >= tn_up;
+                t.dep = t.kind == 0 ? 0u : atomic_load_relaxed(rd.counter(t));
+                t.ready = t.kind == 0 || rd.complete(t.dep);
                 t.valid = 1;
                 break;
             }
@@ -449,11 +510,11 @@ __global__ __launch_bounds__(TileShape<T>::kThreads, TileShape<T>::kPerCu) void 
     };
     expert_loop<T>(p, s_gemm, s_task, rd, stamp + 8, next);
     if (tid == 0) stamp[5] = wall_clock64();
-    grid_barrier(sched, 2, barrier_base + nwg);
+    grid_barrier(sched, 2, seq, nwg);
     if (tid == 0) stamp[6] = wall_clock64();
 
     // ---- phase 3: combine, one token per wavefront
-    for (uint32_t token = blockIdx.x * kWaves + wave; token < p.S; token += nwg * kWaves) combine_token<T>(p, token);
+    combine_tokens<T>(p, blockIdx.x * kWaves + wave, nwg * kWaves);
     __syncthreads();
     if (tid == 0) stamp[7] = wall_clock64();
 }
@@ -589,11 +650,10 @@ hipError_t plan_fused(const LayerParams& p, int dtype, int num_cus, FusedPlan* p
 }
 
 hipError_t launch_fused(const LayerParams& p, const FusedPlan& plan, uint32_t fused_seq, hipStream_t s) {
-    // arrivals recorded on the barrier counters by earlier fused launches (mod 2^32)
-    uint32_t barrier_base = fused_seq * plan.nwg;
+    uint32_t seq = fused_seq;
     uint32_t mt_max = plan.mt_max, lag = plan.lag;
     LayerParams pc = p;
-    void* args[] = {&pc, &barrier_base, &mt_max, &lag};
+    void* args[] = {&pc, &seq, &mt_max, &lag};
     return hipLaunchKernel(plan.kernel, dim3(plan.nwg), dim3(plan.threads), args, plan.smem, s);
 }
 

@@ -56,6 +56,15 @@ def scheduler_stats() -> dict:
     return dict(zip(keys, (float(v) for v in arr)))
 
 
+def phase_stamps(max_workgroups: int = 4096) -> np.ndarray:
+    """Raw 100 MHz wall-clock stamps [workgroups, 8] of the last persistent launch. Synchronises."""
+    buf = (C.c_ulonglong * (max_workgroups * 8))()
+    n = C.c_uint32(0)
+    _capi.check(_capi.lib().kleos_phase_stamps(buf, max_workgroups, C.byref(n)))
+    rows = min(int(n.value), max_workgroups)
+    return np.ctypeslib.as_array(buf)[: rows * 8].reshape(rows, 8).copy()
+
+
 def debug_views(derived) -> dict:
     """Copies the routing state of the most recent forward to host numpy arrays. Synchronises."""
     lib = _capi.lib()

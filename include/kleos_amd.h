@@ -171,6 +171,13 @@ int kleos_phase_times(float ms[5]);
  * unfinished dependency, publishing finished tiles; [3] expert tiles executed; [4] tiles handed out
  * before their inputs were complete; [5] tiles taken from another XCD's queue. */
 int kleos_scheduler_stats(double stats[6]);
+/* Raw phase stamps of the most recent persistent launch (KLEOS_MODE_FUSED), for timing studies; the
+ * reference has no counterpart. Synchronises the library stream, then copies, for each of the first
+ * min(*n_workgroups, max_workgroups) workgroups, 8 readings of the 100 MHz device wall clock:
+ * [0] kernel entry, [1] gate tiles done, [2] past barrier 1, [3] slots done, [4] past barrier 2,
+ * [5] expert tiles done, [6] past barrier 3, [7] combine done. *n_workgroups receives the size of
+ * the launch. */
+int kleos_phase_stamps(unsigned long long* stamps, uint32_t max_workgroups, uint32_t* n_workgroups);
 
 /* ---- errors --------------------------------------------------------------------------------- */
 /* Replaces the KLEOS_CHECK_CUDA / KLEOS_ASSERT message conventions (csrc/include/kleos/debug.cuh:

@@ -214,6 +214,68 @@ def test_back_to_back_launches_need_no_host_reset(mode):
     np.testing.assert_array_equal(v5["topk_slot"], v1["topk_slot"])
 
 
+@pytest.mark.parametrize("mode", MODES, ids=MODE_IDS)
+def test_new_inputs_in_the_same_context(mode):
+    """Routing tables, h1 and y of one launch must not leak into the next: three different batches
+    (different routing, different drops) run through one context, each checked against the oracle.
+    Every table that crosses workgroups is rewritten by other CUs and XCDs than the ones that read
+    it last time, which is what a stale cache line would show up in."""
+    keys = _keys(1024, 128, 256, 24, 2)
+    c = moe_ref.cfg_from_keys(keys)
+    d = ka.initialize(keys)
+    try:
+        ka.moe.set_mode(mode)
+        oP = synth.alloc_outputs(d)
+        for seed in (21, 22, 23):
+            x, wg, w_up, w_down, *_ = random_layer(c, seed=seed, w_std=0.3 if seed == 22 else 0.08)
+            iP_np = pack_inputs(c, x, wg, w_up, w_down)
+            iP = _to_device(c, iP_np)
+            oP.fill_(float("nan"))
+            torch.cuda.synchronize()
+            ka.moe.forward_host(iP, oP)
+            ka.moe.forward_host(iP, oP)
+            ka.moe.stream_synchronize()
+            v = ka.moe.debug_views(d)
+            ref = moe_ref.forward(c, iP_np, logits=v["logits"])
+            for name in ("topk_expert", "topk_slot", "expert_count"):
+                np.testing.assert_array_equal(v[name], ref[name], err_msg=f"{name}, seed {seed}")
+            out = moe_ref.elems_to_f32(_out_to_np(c, oP), c)
+            assert np.isfinite(out).all()
+            moe_out = out[c.S * c.PX:].reshape(c.S, c.H)
+            assert rel_fro(moe_out, ref["moe_out"]) < TOL_OUT[c.dtype], f"seed {seed}"
+    finally:
+        ka.finalize()
+
+
+def test_timing_interfaces_of_the_persistent_launch():
+    """kleos_phase_times, kleos_scheduler_stats and kleos_phase_stamps after a fused bench run: the
+    stamps are monotonic per workgroup, every expert tile is counted once, phases add up to less
+    than the event-timed launch."""
+    keys = _keys(2048, 512, 512, 16, 2)
+    c = moe_ref.cfg_from_keys(keys)
+    x, wg, w_up, w_down, *_ = random_layer(c, seed=31, w_std=0.05)
+    iP = _to_device(c, pack_inputs(c, x, wg, w_up, w_down))
+    d = ka.initialize(keys)
+    try:
+        ka.moe.set_mode(ka.MODE_FUSED)
+        oP = synth.alloc_outputs(d)
+        ms = ka.moe.forward_host_bench(iP, oP, skip=2, trials=4)
+        ph = ka.moe.phase_times()
+        st = ka.moe.scheduler_stats()
+        stamps = ka.moe.phase_stamps()
+        v = ka.moe.debug_views(d)
+    finally:
+        ka.finalize()
+    assert ms > 0 and all(t >= 0 for t in ph.values())
+    assert sum(ph.values()) <= ms * 1.5 + 0.05
+    assert stamps.shape[1] == 8 and stamps.shape[0] >= 1
+    assert (np.diff(stamps.astype(np.int64), axis=1) >= 0).all()
+    kept = np.minimum(v["expert_count"].astype(np.int64), d.kept_capacity)
+    row_blocks = -(-kept // 256)
+    assert int(st["tiles"]) == int(row_blocks.sum()) * (-(-d.I // 256) + -(-d.H // 256))
+    assert st["foreign_tiles"] <= st["tiles"]
+
+
 def test_fused_and_phased_agree_bitwise():
     keys = _keys(1024, 256, 256, 16, 2)
     c = moe_ref.cfg_from_keys(keys)
