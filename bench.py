@@ -22,6 +22,11 @@ sys.path.insert(0, ROOT)
 PEAK_BF16_TFLOPS = 2500.0     # MI355X dense bf16 MFMA
 PEAK_FP32_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
+# HBM bytes per launch of the persistent kernel, from the two rocprofv3 --pmc passes (FETCH_SIZE,
+# WRITE_SIZE, each scaled by what the counter reads for a 1 GiB copy) summarised in
+# profiles/fused_kernel_headline_e64_zipf_hbm_traffic.txt. Counters cannot be read inside a timed
+# run, so the figure is carried here; --traffic-bytes overrides it after a new pair of passes.
+MEASURED_TRAFFIC_BYTES = {"headline_e64_zipf": 1.4171e9}
 
 
 def main() -> int:
@@ -39,6 +44,8 @@ def main() -> int:
                     help="measured HBM bytes per launch of the persistent kernel (from the rocprofv3 --pmc runs "
                          "recorded under profiles/), reported as roofline.traffic")
     args = ap.parse_args()
+    if args.traffic_bytes is None:
+        args.traffic_bytes = MEASURED_TRAFFIC_BYTES.get(args.workload)
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures the single-GPU path (expert-parallel degree 1) only; run it with --gpus 1",
               file=sys.stderr)
