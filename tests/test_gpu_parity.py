@@ -326,3 +326,21 @@ def test_headline_e64_zipf_full_size(mode):
     assert 3.5 * mean < counts.max() < 4.6 * mean, counts.max() / mean
     assert (v["topk_slot"] < 0).sum() > 0
     assert (np.minimum(counts, c.EC).sum()) == (v["topk_slot"] >= 0).sum()
+
+
+@pytest.mark.parametrize("mode", MODES, ids=MODE_IDS)
+def test_mixtral_e8_full_size(mode):
+    """S=8192 H=4096 I=14336 E=8 top-2 cf=1.25 bf16: large, compute-bound expert GEMMs with several
+    row blocks per expert; the oracle evaluates a sample of the tokens."""
+    c, w, iP_np, mask = _full_size("mixtral_e8", mode, 48)
+    d, v, moe_out, err = check_against_oracle(c, w.config, iP_np, mode, token_mask=mask)
+    assert v["expert_count"].astype(np.int64).sum() == c.S * c.k
+
+
+@pytest.mark.parametrize("mode", MODES, ids=MODE_IDS)
+def test_fine_e256_top8_full_size(mode):
+    """S=4096 H=7168 I=2048 E=256 top-8 bf16: many small experts, dispatch / combine / scheduler
+    dominated."""
+    c, w, iP_np, mask = _full_size("fine_e256_top8", mode, 48)
+    d, v, moe_out, err = check_against_oracle(c, w.config, iP_np, mode, token_mask=mask)
+    assert v["expert_count"].astype(np.int64).sum() == c.S * c.k
