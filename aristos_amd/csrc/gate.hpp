@@ -23,202 +23,242 @@ struct GateK {
     static constexpr int kStepK = 4 * kElemsPer16B;
 };
 
-// LDS floats needed by gate_tile: three partial accumulators of 4*NG registers for 64 lanes.
+// Token blocks (16 tokens each) one gate unit works on together: the fragments of the gate weights
+// are loaded once per unit and used by every block, which halves the L2 traffic of the weights.
+// With 16 expert groups (E > 128) the accumulators of two blocks no longer fit the register file.
 template <int NG>
-constexpr int gate_smem_floats() { return 3 * NG * 4 * kWave; }
+constexpr int gate_unit_blocks() { return NG >= 16 ? 1 : 2; }
 
-// One 16-token tile of the gate, computed by a group of four wavefronts (256 threads): the four
-// waves split the hidden dimension, wave 0 of the group reduces the partial sums in a fixed order
-// and runs the epilogue. A workgroup of 256*G threads runs G groups side by side on different
-// tiles; every thread of the workgroup must call the function (it contains workgroup barriers) and
-// a group without a tile passes valid = false. `smem` is the group's private scratch of
-// gate_smem_floats<NG>() floats; it may be reused after the call (which ends with a barrier).
+// LDS floats needed by gate_unit with KW wavefronts: the partial accumulators (4*NG registers of
+// 64 lanes) of the KW-1 wavefronts that do not own the block being reduced.
+template <int NG>
+constexpr int gate_smem_floats(int kw) { return (kw - 1) * NG * 4 * kWave; }
+
+// Softmax, top-k, outputs and the tile histogram of one 16-token tile, run by one wavefront that
+// holds the complete logits of the tile: acc[g][v] of lane l is expert 16 g + 4 (l / 16) + v of
+// token l % 16.
 template <typename T, int NG>
-__device__ __forceinline__ void gate_tile(const LayerParams& p, uint32_t tile, bool valid, float* smem) {
-    const int tid = threadIdx.x & 255;
-    const int wave = tid >> 6, lane = tid & 63;
-    const int col = lane & 15;       // token inside the tile / expert row inside a group
-    const int chunk = lane >> 4;     // which 16-byte K chunk of a step this lane loads
-    const uint32_t H = p.H, E = p.E;
+__device__ __forceinline__ void gate_epilogue(const LayerParams& p, uint32_t tile, f32x4 (&acc)[NG], int lane) {
+    const int col = lane & 15, chunk = lane >> 4;
+    const uint32_t E = p.E;
     const uint32_t token = tile * kGateTileTokens + col;
+    // This lane holds, for its token, experts e = 16 g + 4 chunk + v. The logits stay in the
+    // accumulator registers (padded experts set to -inf); probabilities are recomputed where they
+    // are needed rather than kept, and the selection rounds are packed two to a register: with 16
+    // expert groups there is no room for three more arrays of the accumulator's size.
+    const float kNegInf = -__builtin_inff();
+    float m = kNegInf;
+#pragma unroll
+    for (int g = 0; g < NG; ++g)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const uint32_t e = 16 * g + 4 * chunk + v;
+            if (e < E) p.logits[size_t(token) * E + e] = acc[g][v];
+            // softmax domain = the E real experts only (gate.cuh:550)
+            else acc[g][v] = kNegInf;
+            m = fmaxf(m, acc[g][v]);
+        }
+    m = fmaxf(m, __shfl_xor(m, 16));
+    m = fmaxf(m, __shfl_xor(m, 32));
+    float d = 0.f;
+#pragma unroll
+    for (int g = 0; g < NG; ++g)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) d += __expf(acc[g][v] - m);   // exp(-inf) = 0 for padded experts
+    d += __shfl_xor(d, 16);
+    d += __shfl_xor(d, 32);
+    const float inv_d = 1.0f / d;
+    auto prob = [&](float logit) { return __expf(logit - m) * inv_d; };
+    T* grow = static_cast<T*>(p.gate_out) + size_t(token) * p.PX;
+#pragma unroll
+    for (int g = 0; g < NG; ++g)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const uint32_t e = 16 * g + 4 * chunk + v;
+            // gateOut[t, e] = Element(p) (gate.cuh:590-605); padded columns are zero
+            if (e < p.PX) grow[e] = float_to_elem<T>(e < E ? prob(acc[g][v]) : 0.f);
+        }
+    for (uint32_t e = 16 * NG + 4 * chunk; e < p.PX; e += 16) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v)
+            if (e + v < p.PX) grow[e + v] = float_to_elem<T>(0.f);
+    }
+
+    // top-k: k rounds of arg-max, equal values go to the lower expert index (gate.cuh:654-670).
+    // picked[g][v / 2] holds, in the 16-bit half v % 2, 1 + the round that selected the expert.
+    uint32_t picked[NG][2];
+#pragma unroll
+    for (int g = 0; g < NG; ++g) picked[g][0] = picked[g][1] = 0u;
+    auto round_of = [&](int g, int v) { return (picked[g][v >> 1] >> (16 * (v & 1))) & 0xffffu; };
+    float den = 0.f;
+    constexpr uint32_t kNone = 0x7fffffffu;
+    for (uint32_t r = 0; r < p.k; ++r) {
+        float best = kNegInf;
+        uint32_t bi = kNone;
+#pragma unroll
+        for (int g = 0; g < NG; ++g)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const uint32_t e = 16 * g + 4 * chunk + v;
+                // padded experts hold -inf and can never beat the initial best
+                if (round_of(g, v) == 0 && acc[g][v] > best) {
+                    best = acc[g][v];
+                    bi = e;
+                }
+            }
+#pragma unroll
+        for (int off = 16; off <= 32; off <<= 1) {
+            const float ob = __shfl_xor(best, off);
+            const uint32_t oi = __shfl_xor(bi, off);
+            if (oi != kNone && (bi == kNone || ob > best || (ob == best && oi < bi))) {
+                best = ob;
+                bi = oi;
+            }
+        }
+        float pv = 0.f;
+#pragma unroll
+        for (int g = 0; g < NG; ++g)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const uint32_t e = 16 * g + 4 * chunk + v;
+                if (e == bi) {
+                    picked[g][v >> 1] |= (r + 1u) << (16 * (v & 1));
+                    pv = prob(acc[g][v]);
+                }
+            }
+        // exactly one of the four lanes of this token holds the winner; the others add 0
+        pv += __shfl_xor(pv, 16);
+        pv += __shfl_xor(pv, 32);
+        den += pv;   // mCw, accumulated in selection order (gate.cuh:669)
+        if (chunk == 0) {
+            p.topk_expert[size_t(token) * p.k + r] = int32_t(bi);
+            p.topk_prob[size_t(token) * p.k + r] = pv;
+        }
+    }
+    if (chunk == 0) p.combine_den[token] = den;
+
+    // Histogram of the tile and each token's rank inside it (gate.cuh:678-696).
+    uint32_t* super = p.super_count + size_t(p.epoch & 1u) * p.n_super * E +
+                      size_t(tile / kSuperTiles) * E;
+#pragma unroll
+    for (int g = 0; g < NG; ++g)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const uint32_t e = 16 * g + 4 * chunk + v;
+            const uint32_t rnd = round_of(g, v);
+            const bool sel = rnd != 0;
+            const unsigned long long mask = __ballot(sel);
+            const uint32_t sub = uint32_t(mask >> (16 * chunk)) & 0xffffu;
+            if (sel)
+                p.topk_slot[size_t(token) * p.k + (rnd - 1)] = int32_t(__popc(sub & ((1u << col) - 1u)));
+            if (col == 0 && e < E) {
+                const uint32_t cnt = __popc(sub);
+                p.tile_count[size_t(tile) * E + e] = cnt;
+                if (cnt) atomic_add_agent(super + e, cnt);
+            }
+        }
+}
+
+// One gate unit: gate_unit_blocks<NG>() consecutive 16-token tiles, computed by the KW wavefronts of the
+// workgroup, which split the hidden dimension. Wavefront b then reduces the partial sums of block
+// b in a fixed order and runs its epilogue. Every thread of the workgroup must call the function
+// (it contains workgroup barriers); `smem` holds gate_smem_floats<NG>(KW) floats and may be reused
+// after the call.
+template <typename T, int NG, int KW>
+__device__ __forceinline__ void gate_unit(const LayerParams& p, uint32_t unit, float* smem) {
+    constexpr int TB = gate_unit_blocks<NG>();
+    static_assert(TB <= KW);
+    const int wave = __builtin_amdgcn_readfirstlane(int(threadIdx.x >> 6)), lane = threadIdx.x & 63;
+    const int col = lane & 15;       // token inside a block / expert row inside a group
+    const int chunk = lane >> 4;     // which 16-byte K chunk of a step this lane loads
+    const uint32_t H = p.H;
     constexpr int kStepK = GateK<T>::kStepK;
     constexpr int kPer = GateK<T>::kElemsPer16B;
-
     const uint32_t steps = H / kStepK;
-    const uint32_t s0 = (steps * wave) / 4, s1 = (steps * (wave + 1)) / 4;
+    const uint32_t s0 = (steps * wave) / KW, s1 = (steps * (wave + 1)) / KW;
 
-    const T* xrow = static_cast<const T*>(p.x) + size_t(token) * H + chunk * kPer;
+    const T* xrow[TB];
+    bool live[TB];
+#pragma unroll
+    for (int b = 0; b < TB; ++b) {
+        const uint32_t tile = unit * TB + b;
+        live[b] = tile < p.n_gate_tiles;
+        // a block past the end re-reads the last tile; nothing of it is written
+        const uint32_t token = (live[b] ? tile : p.n_gate_tiles - 1) * kGateTileTokens + col;
+        xrow[b] = static_cast<const T*>(p.x) + size_t(token) * H + chunk * kPer;
+    }
     const T* wrow = static_cast<const T*>(p.wg) + size_t(col) * H + chunk * kPer;
 
-    f32x4 acc[NG];
+    f32x4 acc[TB][NG];
 #pragma unroll
-    for (int g = 0; g < NG; ++g) acc[g] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int b = 0; b < TB; ++b)
+#pragma unroll
+        for (int g = 0; g < NG; ++g) acc[b][g] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    // logits^T tile: experts are the matrix-core rows, tokens its columns (gate.cuh:526-534).
-    // The loads of U steps are issued together before their matrix instructions: the activation
-    // rows stream from HBM once and this is what keeps enough of them in flight.
-    constexpr int U = NG <= 4 ? 4 : (NG <= 8 ? 2 : 1);
-    uint32_t s = valid ? s0 : s1;
+    // logits^T: experts are the matrix-core rows, tokens its columns (gate.cuh:526-534). The loads
+    // of U steps are issued together before their matrix instructions: the activation rows stream
+    // from HBM once and this is what keeps enough of them in flight.
+    constexpr int U = NG <= 2 ? 8 : (NG <= 4 ? 4 : (NG <= 8 ? 2 : 1));
+    uint32_t s = s0;
     for (; s + U <= s1; s += U) {
-        u32x4 b[U], a[U][NG];
+        u32x4 xb[U][TB], wa[U][NG];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const uint32_t off = (s + u) * kStepK;
-            b[u] = load16(xrow + off);
 #pragma unroll
-            for (int g = 0; g < NG; ++g) a[u][g] = load16(wrow + size_t(g) * 16 * H + off);
+            for (int b = 0; b < TB; ++b) xb[u][b] = load16(xrow[b] + off);
+#pragma unroll
+            for (int g = 0; g < NG; ++g) wa[u][g] = load16(wrow + size_t(g) * 16 * H + off);
         }
+        // every load above is issued before the first matrix instruction waits for one of them
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int u = 0; u < U; ++u)
 #pragma unroll
-            for (int g = 0; g < NG; ++g) acc[g] = mma16_step(a[u][g], b[u], acc[g], T{});
+            for (int g = 0; g < NG; ++g)
+#pragma unroll
+                for (int b = 0; b < TB; ++b) acc[b][g] = mma16_step(wa[u][g], xb[u][b], acc[b][g], T{});
     }
     for (; s < s1; ++s) {
         const uint32_t off = s * kStepK;
-        const u32x4 b = load16(xrow + off);
+        u32x4 xb[TB];
+#pragma unroll
+        for (int b = 0; b < TB; ++b) xb[b] = load16(xrow[b] + off);
 #pragma unroll
         for (int g = 0; g < NG; ++g) {
             const u32x4 a = load16(wrow + size_t(g) * 16 * H + off);
-            acc[g] = mma16_step(a, b, acc[g], T{});
+#pragma unroll
+            for (int b = 0; b < TB; ++b) acc[b][g] = mma16_step(a, xb[b], acc[b][g], T{});
         }
     }
 
-    if (valid && wave > 0) {
-        float* dst = smem + (wave - 1) * (NG * 4 * kWave);
+    // Block b: every wavefront but b parks its partial sums in LDS, wavefront b adds them to its
+    // own in ascending wavefront order (a fixed order: the logits do not depend on timing).
 #pragma unroll
-        for (int g = 0; g < NG; ++g)
+    for (int b = 0; b < TB; ++b) {
+        if (wave != b) {
+            float* dst = smem + (wave - (wave > b ? 1 : 0)) * (NG * 4 * kWave);
 #pragma unroll
-            for (int v = 0; v < 4; ++v) dst[(g * 4 + v) * kWave + lane] = acc[g][v];
+            for (int g = 0; g < NG; ++g)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) dst[(g * 4 + v) * kWave + lane] = acc[b][g][v];
+        }
+        __syncthreads();
+        if (wave == b) {
+#pragma unroll
+            for (int w = 0; w < KW - 1; ++w) {
+                const float* src = smem + w * (NG * 4 * kWave);
+#pragma unroll
+                for (int g = 0; g < NG; ++g)
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) acc[b][g][v] += src[(g * 4 + v) * kWave + lane];
+            }
+        }
+        __syncthreads();
     }
-    __syncthreads();
-    if (valid && wave == 0) {
-        // fixed summation order: wave 0 + wave 1 + wave 2 + wave 3
 #pragma unroll
-        for (int w = 0; w < 3; ++w) {
-            const float* src = smem + w * (NG * 4 * kWave);
-#pragma unroll
-            for (int g = 0; g < NG; ++g)
-#pragma unroll
-                for (int v = 0; v < 4; ++v) acc[g][v] += src[(g * 4 + v) * kWave + lane];
-        }
-
-        // This lane holds, for its token, experts e = 16 g + 4 chunk + v.
-        const float kNegInf = -__builtin_inff();
-        float lg[NG][4];
-        float m = kNegInf;
-#pragma unroll
-        for (int g = 0; g < NG; ++g)
-#pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                const uint32_t e = 16 * g + 4 * chunk + v;
-                // softmax domain = the E real experts only (gate.cuh:550)
-                lg[g][v] = e < E ? acc[g][v] : kNegInf;
-                if (e < E) p.logits[size_t(token) * E + e] = acc[g][v];
-                m = fmaxf(m, lg[g][v]);
-            }
-        m = fmaxf(m, __shfl_xor(m, 16));
-        m = fmaxf(m, __shfl_xor(m, 32));
-        float d = 0.f;
-        float pr[NG][4];
-#pragma unroll
-        for (int g = 0; g < NG; ++g)
-#pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                pr[g][v] = __expf(lg[g][v] - m);   // exp(-inf) = 0 for padded experts
-                d += pr[g][v];
-            }
-        d += __shfl_xor(d, 16);
-        d += __shfl_xor(d, 32);
-        const float inv_d = 1.0f / d;
-        T* grow = static_cast<T*>(p.gate_out) + size_t(token) * p.PX;
-#pragma unroll
-        for (int g = 0; g < NG; ++g)
-#pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                const uint32_t e = 16 * g + 4 * chunk + v;
-                pr[g][v] *= inv_d;
-                // gateOut[t, e] = Element(p) (gate.cuh:590-605); padded columns are zero
-                if (e < p.PX) grow[e] = float_to_elem<T>(e < E ? pr[g][v] : 0.f);
-            }
-        for (uint32_t e = 16 * NG + 4 * chunk; e < p.PX; e += 16) {
-#pragma unroll
-            for (int v = 0; v < 4; ++v)
-                if (e + v < p.PX) grow[e + v] = float_to_elem<T>(0.f);
-        }
-
-        // top-k: k rounds of arg-max, equal values go to the lower expert index (gate.cuh:654-670).
-        int sel_round[NG][4];
-#pragma unroll
-        for (int g = 0; g < NG; ++g)
-#pragma unroll
-            for (int v = 0; v < 4; ++v) sel_round[g][v] = -1;
-        float den = 0.f;
-        constexpr uint32_t kNone = 0x7fffffffu;
-        for (uint32_t r = 0; r < p.k; ++r) {
-            float best = kNegInf;
-            uint32_t bi = kNone;
-#pragma unroll
-            for (int g = 0; g < NG; ++g)
-#pragma unroll
-                for (int v = 0; v < 4; ++v) {
-                    const uint32_t e = 16 * g + 4 * chunk + v;
-                    if (e < E && sel_round[g][v] < 0 && (bi == kNone || lg[g][v] > best)) {
-                        best = lg[g][v];
-                        bi = e;
-                    }
-                }
-#pragma unroll
-            for (int off = 16; off <= 32; off <<= 1) {
-                const float ob = __shfl_xor(best, off);
-                const uint32_t oi = __shfl_xor(bi, off);
-                if (oi != kNone && (bi == kNone || ob > best || (ob == best && oi < bi))) {
-                    best = ob;
-                    bi = oi;
-                }
-            }
-            float pv = 0.f;
-#pragma unroll
-            for (int g = 0; g < NG; ++g)
-#pragma unroll
-                for (int v = 0; v < 4; ++v) {
-                    const uint32_t e = 16 * g + 4 * chunk + v;
-                    if (e == bi) {
-                        sel_round[g][v] = int(r);
-                        pv = pr[g][v];
-                    }
-                }
-            // exactly one of the four lanes of this token holds the winner; the others add 0
-            pv += __shfl_xor(pv, 16);
-            pv += __shfl_xor(pv, 32);
-            den += pv;   // mCw, accumulated in selection order (gate.cuh:669)
-            if (chunk == 0) {
-                p.topk_expert[size_t(token) * p.k + r] = int32_t(bi);
-                p.topk_prob[size_t(token) * p.k + r] = pv;
-            }
-        }
-        if (chunk == 0) p.combine_den[token] = den;
-
-        // Histogram of the tile and each token's rank inside it (gate.cuh:678-696).
-        uint32_t* super = p.super_count + size_t(p.epoch & 1u) * p.n_super * E +
-                          size_t(tile / kSuperTiles) * E;
-#pragma unroll
-        for (int g = 0; g < NG; ++g)
-#pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                const uint32_t e = 16 * g + 4 * chunk + v;
-                const bool sel = sel_round[g][v] >= 0;
-                const unsigned long long mask = __ballot(sel);
-                const uint32_t sub = uint32_t(mask >> (16 * chunk)) & 0xffffu;
-                if (sel)
-                    p.topk_slot[size_t(token) * p.k + sel_round[g][v]] =
-                        int32_t(__popc(sub & ((1u << col) - 1u)));
-                if (col == 0 && e < E) {
-                    const uint32_t cnt = __popc(sub);
-                    p.tile_count[size_t(tile) * E + e] = cnt;
-                    if (cnt) atomic_add_agent(super + e, cnt);
-                }
-            }
-    }
+    for (int b = 0; b < TB; ++b)
+        if (wave == b && live[b]) gate_epilogue<T, NG>(p, unit * TB + b, acc[b], lane);
     __syncthreads();
 }
 

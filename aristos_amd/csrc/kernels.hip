@@ -319,10 +319,13 @@ __device__ __forceinline__ void expert_loop(const LayerParams& p, char* smem, ui
 }
 
 // ------------------------------------------------------------------------------------ phased
+// One gate unit per workgroup, with as many wavefronts as the persistent kernel's workgroups have:
+// the split of the hidden dimension, and with it the summation order of the logits, is the same
+// in both modes.
 template <typename T, int NG>
-__global__ __launch_bounds__(kPhaseThreads) void gate_kernel(const LayerParams p) {
-    __shared__ float smem[gate_smem_floats<NG>()];
-    gate_tile<T, NG>(p, blockIdx.x, true, smem);
+__global__ __launch_bounds__(TileShape<T>::kThreads) void gate_kernel(const LayerParams p) {
+    extern __shared__ __attribute__((aligned(16))) float gate_smem[];
+    gate_unit<T, NG, TileShape<T>::kThreads / kWave>(p, blockIdx.x, gate_smem);
 }
 
 __global__ __launch_bounds__(kPhaseThreads) void slot_kernel(const LayerParams p) {
@@ -401,9 +404,8 @@ __global__ __launch_bounds__(TileShape<T>::kThreads, TileShape<T>::kPerCu) void 
         if (tid < uint32_t(kXcds)) sched[kSchedTicket + tid * kSchedLine] = 0u;
         for (uint32_t i = tid; i < p.E * mt_max; i += kThreads) sched[kSchedReady + i] = 0u;
     }
-    for (uint32_t t0 = blockIdx.x * kGroups; t0 < p.n_gate_tiles; t0 += nwg * kGroups)
-        gate_tile<T, NG>(p, t0 + group, t0 + group < p.n_gate_tiles,
-                         reinterpret_cast<float*>(smem) + group * gate_smem_floats<NG>());
+    for (uint32_t unit = blockIdx.x; unit < ceil_div_u32(p.n_gate_tiles, gate_unit_blocks<NG>()); unit += nwg)
+        gate_unit<T, NG, int(kWaves)>(p, unit, reinterpret_cast<float*>(smem));
     if (tid == 0) stamp[1] = wall_clock64();
     grid_barrier(sched, 0, seq, nwg);
     if (tid == 0) stamp[2] = wall_clock64();
@@ -522,7 +524,7 @@ __global__ __launch_bounds__(TileShape<T>::kThreads, TileShape<T>::kPerCu) void 
 template <typename T, int NG>
 size_t fused_smem_bytes(uint32_t E) {
     size_t need = kFusedLdsHeader + gemm_smem_bytes<T>();
-    const size_t gate = (TileShape<T>::kThreads / 256) * gate_smem_floats<NG>() * sizeof(float);
+    const size_t gate = gate_smem_floats<NG>(TileShape<T>::kThreads / kWave) * sizeof(float);
     const size_t slots = (TileShape<T>::kThreads / kWave) * size_t(E) * sizeof(uint32_t);
     if (gate > need) need = gate;
     if (slots > need) need = slots;
@@ -567,9 +569,22 @@ size_t sched_words(uint32_t E, uint32_t cap_rows) {
 hipError_t launch_gate(const LayerParams& p, int dtype, hipStream_t s) {
     return dispatch_groups(p.E, [&](auto ng) {
         constexpr int NG = decltype(ng)::value;
-        if (dtype == 2) hipLaunchKernelGGL((gate_kernel<bf16_t, NG>), dim3(p.n_gate_tiles), dim3(kPhaseThreads), 0, s, p);
-        else hipLaunchKernelGGL((gate_kernel<float, NG>), dim3(p.n_gate_tiles), dim3(kPhaseThreads), 0, s, p);
-        return hipGetLastError();
+        auto go = [&](auto tag) -> hipError_t {
+            using T = decltype(tag);
+            auto kernel = gate_kernel<T, NG>;
+            constexpr int smem = gate_smem_floats<NG>(TileShape<T>::kThreads / kWave) * sizeof(float);
+            static bool prepared = false;   // once per (Element type, group count)
+            if (!prepared && smem > 48 * 1024) {
+                hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+                if (err != hipSuccess) return err;
+            }
+            prepared = true;
+            hipLaunchKernelGGL(kernel, dim3(ceil_div_u32(p.n_gate_tiles, gate_unit_blocks<NG>())), dim3(TileShape<T>::kThreads),
+                               smem, s, p);
+            return hipGetLastError();
+        };
+        return dtype == 2 ? go(bf16_t{}) : go(float{});
     });
 }
 
