@@ -81,11 +81,7 @@ struct GemmBf16 {
     static constexpr int kLoadsPerSlice = LA + LB;                 // per wavefront
     static constexpr int kSteps = BK / 16;                         // matrix instructions consume 16 values of K
     static constexpr int kPanelRows = 32;                          // epilogue staging: 32 rows x 64 columns per wavefront
-#ifdef KLEOS_ISSUE_STEPS
-    static constexpr int kIssueSteps = KLEOS_ISSUE_STEPS;
-#else
     static constexpr int kIssueSteps = kSteps;                     // K steps over which the next slice's loads are issued
-#endif
     static_assert(BK == 32 || BK == 64);
     static_assert(STAGES >= 2 && STAGES <= 4);
     static_assert(WM % 32 == 0 && WN % 64 == 0);
