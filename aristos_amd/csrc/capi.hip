@@ -48,7 +48,7 @@ size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 struct ArenaLayout {
     size_t logits, topk_expert, topk_prob, combine_den, topk_slot, tile_count, super_count,
-        expert_count, slot_token, h1, y, sched, stamps, total;
+        expert_count, slot_token, h1, y, sched, stamps, tile_prob, super_prob, gate_loss, total;
     size_t zero_begin, zero_end;   // range that must start as zeros
 };
 
@@ -63,7 +63,10 @@ ArenaLayout layout_arena(const kleos_config_t& c, uint32_t n_tiles, uint32_t n_s
     L.sched = take(sched_words(c.E, c.cap_rows) * 4);
     L.expert_count = take(E * 4);
     L.stamps = take(size_t(kMaxWorkgroups) * 16 * 8);
+    L.gate_loss = take((2 * E + 1) * 4);
     L.zero_end = off;
+    L.tile_prob = take(size_t(n_tiles) * E * 4);
+    L.super_prob = take(size_t(n_super) * E * 4);
     L.logits = take(S * E * 4);
     L.topk_expert = take(S * k * 4);
     L.topk_prob = take(S * k * 4);
@@ -179,6 +182,7 @@ extern "C" int kleos_initialize_cfg(const kleos_config_t* user_cfg) {
     LayerParams& p = c->base;
     p.S = cfg.S; p.H = cfg.H; p.I = cfg.I; p.E = cfg.E; p.k = cfg.k; p.PX = cfg.PX;
     p.EC = cfg.EC; p.cap_rows = cfg.cap_rows; p.act = cfg.hidden_act;
+    p.is_training = cfg.is_training;
     p.n_gate_tiles = cfg.S / kGateTileTokens;
     p.n_super = (p.n_gate_tiles + kSuperTiles - 1) / kSuperTiles;
     const ArenaLayout L = layout_arena(cfg, p.n_gate_tiles, p.n_super);
@@ -196,6 +200,9 @@ extern "C" int kleos_initialize_cfg(const kleos_config_t* user_cfg) {
     p.super_count = reinterpret_cast<uint32_t*>(a + L.super_count);
     p.expert_count = reinterpret_cast<uint32_t*>(a + L.expert_count);
     p.slot_token = reinterpret_cast<int32_t*>(a + L.slot_token);
+    p.tile_prob = reinterpret_cast<float*>(a + L.tile_prob);
+    p.super_prob = reinterpret_cast<float*>(a + L.super_prob);
+    p.gate_loss = reinterpret_cast<float*>(a + L.gate_loss);
     p.h1 = a + L.h1;
     p.y = a + L.y;
     p.sched = reinterpret_cast<uint32_t*>(a + L.sched);
@@ -363,6 +370,20 @@ extern "C" int kleos_scheduler_stats(double stats[6]) {
     if (!stats) return fail(KLEOS_EINVAL, "kleos_scheduler_stats: null argument");
     for (int i = 0; i < 6; ++i) stats[i] = g_ctx->sched_stats[i];
     return KLEOS_OK;
+}
+
+extern "C" int kleos_gate_loss(float* loss, float* mean_prob, float* mean_count) {
+    if (int rc = require_ctx("kleos_gate_loss")) return rc;
+    Context& c = *g_ctx;
+    if (!c.cfg.is_training) return fail(KLEOS_ESTATE, "kleos_gate_loss: the context was initialised with is_training 0");
+    if (!loss) return fail(KLEOS_EINVAL, "kleos_gate_loss: null argument");
+    KLEOS_HIP(hipSetDevice(c.device));
+    KLEOS_HIP(hipStreamSynchronize(c.stream));
+    const size_t E = c.cfg.E;
+    KLEOS_HIP(hipMemcpy(loss, c.base.gate_loss + 2 * E, 4, hipMemcpyDeviceToHost));
+    if (mean_prob) KLEOS_HIP(hipMemcpy(mean_prob, c.base.gate_loss, E * 4, hipMemcpyDeviceToHost));
+    if (mean_count) KLEOS_HIP(hipMemcpy(mean_count, c.base.gate_loss + E, E * 4, hipMemcpyDeviceToHost));
+    return check_scheduler(c);
 }
 
 extern "C" int kleos_phase_stamps(unsigned long long* stamps, uint32_t max_workgroups, uint32_t* n_workgroups) {

@@ -187,8 +187,6 @@ extern "C" int kleos_config_derive(kleos_config_t* c) {
         return fail(KLEOS_EUNSUPPORTED, "torch_dtype 1 (tf32) is unsupported: CDNA4 has no tf32 matrix path; use 0 (fp32) or 2 (bf16)");
     if (c->torch_dtype == KLEOS_DTYPE_FP16)
         return fail(KLEOS_EUNSUPPORTED, "torch_dtype 3 (fp16) is unsupported in this build; use 0 (fp32) or 2 (bf16)");
-    if (c->is_training)
-        return fail(KLEOS_EUNSUPPORTED, "is_training 1 is unsupported: this build is the inference forward only");
     if (c->num_experts < 1) return fail(KLEOS_EINVAL, "num_experts must be >= 1");
     if (c->num_experts > 65535) return fail(KLEOS_EINVAL, "num_experts must be <= 65535 (types.cuh:479), got %u", c->num_experts);
     if (c->expert_top_k < 1) return fail(KLEOS_EINVAL, "expert_top_k must be >= 1");

@@ -84,6 +84,23 @@ __device__ __forceinline__ void gate_epilogue(const LayerParams& p, uint32_t til
             if (e + v < p.PX) grow[e + v] = float_to_elem<T>(0.f);
     }
 
+    if (p.is_training) {
+        // Column sums of the tile's probabilities for the load-balancing loss (gate.cuh:608-635):
+        // the 16 tokens of an expert sit in 16 consecutive lanes, summed by a fixed xor tree.
+#pragma unroll
+        for (int g = 0; g < NG; ++g)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const uint32_t e = 16 * g + 4 * chunk + v;
+                float col_sum = prob(acc[g][v]);
+                col_sum += __shfl_xor(col_sum, 1);
+                col_sum += __shfl_xor(col_sum, 2);
+                col_sum += __shfl_xor(col_sum, 4);
+                col_sum += __shfl_xor(col_sum, 8);
+                if (col == 0 && e < E) p.tile_prob[size_t(tile) * E + e] = col_sum;
+            }
+    }
+
     // top-k: k rounds of arg-max, equal values go to the lower expert index (gate.cuh:654-670).
     // picked[g][v / 2] holds, in the 16-bit half v % 2, 1 + the round that selected the expert.
     uint32_t picked[NG][2];
@@ -309,6 +326,21 @@ __device__ __forceinline__ void slot_tile(const LayerParams& p, uint32_t tile, b
                 for (uint32_t u = 0; u < kBatch; ++u) acc += r0 + u < n ? v[u] : 0u;
             }
             base[e] = acc;
+            // training: the wavefront of a block's first tile also sums the block's probability rows
+            if (p.is_training && tile == first) {
+                const uint32_t rows = p.n_gate_tiles - first < uint32_t(kSuperTiles) ? p.n_gate_tiles - first
+                                                                                      : uint32_t(kSuperTiles);
+                float total = 0.f;
+                for (uint32_t r0 = 0; r0 < rows; r0 += 16) {
+                    float v[16];
+#pragma unroll
+                    for (uint32_t u = 0; u < 16; ++u)
+                        v[u] = load_coherent(p.tile_prob + size_t(first + (r0 + u < rows ? r0 + u : rows - 1)) * E + e);
+#pragma unroll
+                    for (uint32_t u = 0; u < 16; ++u) total += r0 + u < rows ? v[u] : 0.f;
+                }
+                p.super_prob[size_t(sup) * E + e] = total;
+            }
             // total routed per expert, dropped tokens included (the reference's eC, gate.cuh:699)
             if (tile + 1 == p.n_gate_tiles)
                 p.expert_count[e] = acc + load_coherent(p.tile_count + size_t(tile) * E + e);
@@ -333,6 +365,39 @@ __device__ __forceinline__ void slot_tile(const LayerParams& p, uint32_t tile, b
                    load_coherent(p.topk_slot + size_t(tile) * pairs + i));
     }
     __syncthreads();
+}
+
+// Training mode, one wavefront, after the slot phase has been released: mean probability and mean
+// routed count per expert and their scaled dot product (gate.cuh:763-773). Every sum has a fixed
+// order, so the loss does not depend on timing.
+__device__ __forceinline__ void gate_loss_finalize(const LayerParams& p) {
+    const uint32_t lane = threadIdx.x & 63, E = p.E;
+    const float inv_s = 1.0f / float(p.S);
+    float dot = 0.f;
+    for (uint32_t e0 = 0; e0 < E; e0 += kWave) {
+        const uint32_t e = e0 + lane;
+        float prod = 0.f;
+        if (e < E) {
+            float total = 0.f;
+            for (uint32_t r0 = 0; r0 < p.n_super; r0 += 16) {
+                float v[16];
+#pragma unroll
+                for (uint32_t u = 0; u < 16; ++u)
+                    v[u] = load_coherent(p.super_prob + size_t(r0 + u < p.n_super ? r0 + u : p.n_super - 1) * E + e);
+#pragma unroll
+                for (uint32_t u = 0; u < 16; ++u) total += r0 + u < p.n_super ? v[u] : 0.f;
+            }
+            const float mean_prob = total * inv_s;
+            const float mean_count = float(load_coherent(p.expert_count + e)) * inv_s;
+            p.gate_loss[e] = mean_prob;
+            p.gate_loss[E + e] = mean_count;
+            prod = mean_prob * mean_count;
+        }
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) prod += __shfl_xor(prod, off);
+        dot += prod;
+    }
+    if (lane == 0) p.gate_loss[2 * E] = dot / float(E);
 }
 
 }  // namespace kleos_amd

@@ -379,6 +379,7 @@ __global__ __launch_bounds__(TileShape<T>::kThreads, TileShape<T>::kPerCu) void 
 template <typename T>
 __global__ __launch_bounds__(kPhaseThreads) void combine_kernel(const LayerParams p) {
     const uint32_t token = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (p.is_training && blockIdx.x == gridDim.x - 1 && (threadIdx.x >> 6) == 3) gate_loss_finalize(p);
     combine_tokens<T>(p, token, p.S);
 }
 
@@ -515,6 +516,7 @@ __global__ __launch_bounds__(TileShape<T>::kThreads, TileShape<T>::kPerCu) void 
     if (tid == 0) stamp[6] = wall_clock64();
 
     // ---- phase 3: combine, one token per wavefront
+    if (p.is_training && blockIdx.x == nwg - 1 && wave == kWaves - 1) gate_loss_finalize(p);
     combine_tokens<T>(p, blockIdx.x * kWaves + wave, nwg * kWaves);
     __syncthreads();
     if (tid == 0) stamp[7] = wall_clock64();

@@ -20,6 +20,7 @@ struct TileTask {
 struct LayerParams {
     // ---- configuration (derived as the reference's struct ACC, types.cuh:471-507)
     uint32_t S, H, I, E, k, PX, EC, cap_rows, act;
+    uint32_t is_training;     // 1: the gate also produces its load-balancing loss
     uint32_t n_gate_tiles;    // S / 16
     uint32_t n_super;         // ceil(n_gate_tiles / 32)
     // ---- caller buffers, sliced as moe.cuh:92-98
@@ -41,6 +42,10 @@ struct LayerParams {
     uint32_t* super_count;    // [2][n_super, E]     the same summed over 32 tiles; two epochs
     uint32_t* expert_count;   // [E]
     int32_t* slot_token;      // [E, cap_rows]
+    // ---- training-mode gate loss (reference: gML / gMeC / gL, types.cuh:940-958)
+    float* tile_prob;         // [n_gate_tiles, E]  sum of the tile's 16 probabilities of expert e
+    float* super_prob;        // [n_super, E]       the same summed over 32 tiles
+    float* gate_loss;         // [E] mean probability | [E] mean routed count | [1] loss
     // ---- intermediate activations (reference: xM buffer, types.cuh:976-982)
     void* h1;                 // [E][cap_rows, I]
     void* y;                  // [E][cap_rows, H]

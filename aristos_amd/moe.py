@@ -56,6 +56,16 @@ def scheduler_stats() -> dict:
     return dict(zip(keys, (float(v) for v in arr)))
 
 
+def gate_loss(n_experts: int) -> dict:
+    """Training mode: loss, mean probability [E] and mean routed count [E] of the last forward."""
+    loss = C.c_float(0.0)
+    mp = (C.c_float * n_experts)()
+    mc = (C.c_float * n_experts)()
+    _capi.check(_capi.lib().kleos_gate_loss(C.byref(loss), mp, mc))
+    return {"loss": float(loss.value), "mean_prob": np.array(mp[:], np.float32),
+            "mean_count": np.array(mc[:], np.float32)}
+
+
 def phase_stamps(max_workgroups: int = 4096) -> np.ndarray:
     """Raw 100 MHz wall-clock stamps [workgroups, 8] of the last persistent launch. Synchronises."""
     buf = (C.c_ulonglong * (max_workgroups * 8))()

@@ -171,6 +171,13 @@ int kleos_phase_times(float ms[5]);
  * unfinished dependency, publishing finished tiles; [3] expert tiles executed; [4] tiles handed out
  * before their inputs were complete; [5] tiles taken from another XCD's queue. */
 int kleos_scheduler_stats(double stats[6]);
+/* Training mode (is_training: 1): the load-balancing loss of the gate of the most recent forward,
+ * which the reference leaves in its bookkeeping arena (gML, gMeC, gL; csrc/include/kleos/types.cuh:
+ * 940-958, computed at moe/gate.cuh:608-635, 700-705, 763-773): mean_prob[e] = mean over the tokens
+ * of the softmax probability of expert e, mean_count[e] = tokens routed to e (dropped included) / S,
+ * *loss = sum_e mean_prob[e] * mean_count[e] / E. mean_prob and mean_count ([E] floats) may be
+ * NULL. Synchronises the library stream. KLEOS_ESTATE when the context is not in training mode. */
+int kleos_gate_loss(float* loss, float* mean_prob, float* mean_count);
 /* Raw phase stamps of the most recent persistent launch (KLEOS_MODE_FUSED), for timing studies; the
  * reference has no counterpart. Synchronises the library stream, then copies, for each of the first
  * min(*n_workgroups, max_workgroups) workgroups, 8 readings of the 100 MHz device wall clock:

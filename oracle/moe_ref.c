@@ -24,6 +24,9 @@
  *                        out[t] += Elem(gateOut[t,e]) * Elem(y/combine_den)               mixture, k=1, all-dropped
  *                                                                                           closed forms
  *   zero-initialised output  moe/moe.cuh:43-48
+ *   moe_ref_gate_loss    moe/gate.cuh:608-635 (mean probability per expert), :700-705 (mean    pinned: uniform logits give
+ *                        routed count per expert), :763-773 (loss = sum of products / E)        k / E^2; both means sum to 1
+ *                                                                                               and k; numpy restatement
  *
  * Deliberate, documented choices where the reference is schedule- or hardware-dependent:
  *   - top-k is selected on the fp32 LOGITS (order-equivalent to the probabilities the reference
@@ -80,6 +83,25 @@ static void load_elems(const void* p, size_t off, size_t n, uint32_t dtype, floa
     } else {
         memcpy(dst, (const float*)p + off, n * sizeof(float));
     }
+}
+
+void moe_ref_gate_loss(uint32_t S, uint32_t E, const float* probs, const uint32_t* expert_count,
+                       float* mean_prob, float* mean_count, float* loss) {
+    /* gate.cuh:608-635 adds each tile's column sums of the probabilities, divided by S, into gML;
+     * :700-705 adds each tile's routed counts divided by S into gMeC; :763-773 sums
+     * gML[e] * gMeC[e] / E. The reference's float atomics fix no summation order: sums here are
+     * taken in double and compared within tolerance. */
+    double total = 0.0;
+    for (uint32_t e = 0; e < E; ++e) {
+        double col = 0.0;
+        for (uint32_t t = 0; t < S; ++t) col += (double)probs[(size_t)t * E + e];
+        const double mp = col / (double)S;
+        const double mc = (double)expert_count[e] / (double)S;
+        if (mean_prob) mean_prob[e] = (float)mp;
+        if (mean_count) mean_count[e] = (float)mc;
+        total += mp * mc;
+    }
+    *loss = (float)(total / (double)E);
 }
 
 int moe_ref_threads(void) {

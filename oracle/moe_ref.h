@@ -48,6 +48,12 @@ void moe_ref_slots(uint32_t S, uint32_t E, uint32_t k, uint32_t EC, uint32_t cap
                    const int32_t* topk_expert, int32_t* topk_slot, uint32_t* expert_count,
                    int32_t* slot_token);
 
+/* Training-mode load-balancing loss of the gate: mean_prob[e] = (sum_t probs[t,e]) / S,
+ * mean_count[e] = expert_count[e] / S (all routed tokens, dropped included),
+ * loss = sum_e mean_prob[e] * mean_count[e] / E. mean_prob, mean_count [E] may be NULL. */
+void moe_ref_gate_loss(uint32_t S, uint32_t E, const float* probs, const uint32_t* expert_count,
+                       float* mean_prob, float* mean_count, float* loss);
+
 typedef struct moe_ref_views {
     float* logits;          /* [S,E]   out (or in when logits_given != 0) */
     float* probs;           /* [S,E]   out, fp32 softmax                  */

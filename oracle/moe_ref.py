@@ -60,6 +60,9 @@ def lib() -> C.CDLL:
         h.moe_ref_topk.restype = None
         h.moe_ref_topk.argtypes = [C.c_uint32, C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p,
                                    C.c_void_p, C.c_void_p]
+        h.moe_ref_gate_loss.restype = None
+        h.moe_ref_gate_loss.argtypes = [C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                                        C.c_void_p]
         h.moe_ref_slots.restype = None
         h.moe_ref_slots.argtypes = [C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32, C.c_void_p,
                                     C.c_void_p, C.c_void_p, C.c_void_p]
@@ -150,6 +153,18 @@ def forward(c: RefCfg, iP: np.ndarray, logits: np.ndarray | None = None,
     out["gate_out"] = elems_to_f32(oP[:S * c.PX], c).reshape(S, c.PX)
     out["moe_out"] = elems_to_f32(oP[S * c.PX:], c).reshape(S, c.H)
     return out
+
+
+def gate_loss(c: RefCfg, probs: np.ndarray, expert_count: np.ndarray) -> dict:
+    """Training-mode gate loss from the fp32 softmax probabilities [S,E] and the routed counts [E]."""
+    probs = np.ascontiguousarray(probs, dtype=np.float32).reshape(c.S, c.E)
+    cnt = np.ascontiguousarray(expert_count, dtype=np.uint32).reshape(c.E)
+    mp = np.empty(c.E, np.float32)
+    mc = np.empty(c.E, np.float32)
+    loss = np.empty(1, np.float32)
+    lib().moe_ref_gate_loss(c.S, c.E, probs.ctypes.data, cnt.ctypes.data, mp.ctypes.data, mc.ctypes.data,
+                            loss.ctypes.data)
+    return {"mean_prob": mp, "mean_count": mc, "loss": float(loss[0])}
 
 
 def route(c: RefCfg, logits: np.ndarray) -> dict:

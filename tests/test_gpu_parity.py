@@ -344,3 +344,50 @@ def test_fine_e256_top8_full_size(mode):
     c, w, iP_np, mask = _full_size("fine_e256_top8", mode, 48)
     d, v, moe_out, err = check_against_oracle(c, w.config, iP_np, mode, token_mask=mask)
     assert v["expert_count"].astype(np.int64).sum() == c.S * c.k
+
+
+# ------------------------------------------------------------------ training mode
+@pytest.mark.parametrize("E,k,S", [(16, 2, 1024), (64, 2, 2048), (130, 8, 512)])
+def test_training_mode_gate_loss(E, k, S):
+    """is_training: 1 adds the load-balancing loss of the gate (gate.cuh:608-635, 700-705, 763-773):
+    checked against the oracle evaluated on the GPU's own logits, identical in both modes (every
+    sum has a fixed order), and the forward itself is unchanged."""
+    keys = _keys(S, 128, 128, E, k)
+    keys.is_training = 1
+    c = moe_ref.cfg_from_keys(keys)
+    x, wg, w_up, w_down, *_ = random_layer(c, seed=41, w_std=0.25)
+    iP_np = pack_inputs(c, x, wg, w_up, w_down)
+    iP = _to_device(c, iP_np)
+    got = {}
+    for mode in MODES:
+        d = ka.initialize(keys)
+        try:
+            ka.moe.set_mode(mode)
+            oP = synth.alloc_outputs(d)
+            ka.moe.forward_host(iP, oP)
+            ka.moe.forward_host(iP, oP)
+            ka.moe.stream_synchronize()
+            got[mode] = (ka.moe.gate_loss(d.E), ka.moe.debug_views(d), _out_to_np(c, oP))
+        finally:
+            ka.finalize()
+    g, v, out = got[ka.MODE_FUSED]
+    r = moe_ref.route(c, v["logits"])
+    np.testing.assert_array_equal(v["expert_count"], r["expert_count"])
+    ref = moe_ref.gate_loss(c, r["probs"], r["expert_count"])
+    assert abs(g["loss"] - ref["loss"]) < 2e-5 * ref["loss"] + 1e-9, (g["loss"], ref["loss"])
+    np.testing.assert_allclose(g["mean_prob"], ref["mean_prob"], rtol=2e-5, atol=1e-8)
+    np.testing.assert_allclose(g["mean_count"], ref["mean_count"], rtol=1e-6, atol=0)
+    gp, vp, outp = got[ka.MODE_PHASED]
+    assert gp["loss"] == g["loss"]
+    np.testing.assert_array_equal(gp["mean_prob"], g["mean_prob"])
+    np.testing.assert_array_equal(outp, out)
+
+
+def test_gate_loss_needs_training_mode():
+    keys = _keys(256, 128, 128, 8, 2)
+    d = ka.initialize(keys)
+    try:
+        with pytest.raises(ka.KleosError):
+            ka.moe.gate_loss(d.E)
+    finally:
+        ka.finalize()

@@ -285,3 +285,41 @@ def test_given_logits_drive_the_routing(oracle):
     np.testing.assert_array_equal(flipped["topk_expert"], npr.topk_lowest_index_first(-base["logits"], 2))
     same = oracle.forward(c, iP, logits=base["logits"])
     np.testing.assert_array_equal(same["oP"], base["oP"])
+
+
+# ------------------------------------------------------------------ training-mode gate loss
+def test_gate_loss_uniform_logits_closed_form(oracle):
+    """Equal logits: every probability is 1/E, so loss = sum_e (1/E)(c_e/S)/E = k/E^2 whatever the
+    routing does (the counts sum to S*k)."""
+    for S, E, k in ((256, 8, 2), (128, 64, 8), (384, 24, 3)):
+        c = oracle.make_cfg(S=S, H=64, I=64, E=E, k=k, dtype=0)
+        r = oracle.route(c, np.zeros((S, E), np.float32))
+        g = oracle.gate_loss(c, r["probs"], r["expert_count"])
+        assert abs(g["loss"] - k / E**2) < 1e-7
+        np.testing.assert_allclose(g["mean_prob"], 1.0 / E, rtol=1e-6)
+        # ties go to the lowest indices: the first k experts take every token
+        np.testing.assert_allclose(g["mean_count"][:k], 1.0, rtol=0, atol=0)
+        assert (g["mean_count"][k:] == 0).all()
+
+
+def test_gate_loss_vs_numpy_and_invariants(oracle):
+    rng = np.random.default_rng(17)
+    S, E, k = 512, 48, 4
+    c = oracle.make_cfg(S=S, H=64, I=64, E=E, k=k, dtype=0)
+    logits = (rng.standard_normal((S, E)) * 2.0).astype(np.float32)
+    r = oracle.route(c, logits)
+    g = oracle.gate_loss(c, r["probs"], r["expert_count"])
+    # independent: float64 softmax, counts from a brute-force top-k
+    l64 = logits.astype(np.float64)
+    p = np.exp(l64 - l64.max(1, keepdims=True)); p /= p.sum(1, keepdims=True)
+    te = npr.topk_lowest_index_first(logits, k)
+    counts = np.bincount(te.ravel(), minlength=E)
+    expect = float((p.mean(0) * counts / S).sum() / E)
+    assert abs(g["loss"] - expect) < 1e-6 * max(1.0, expect)
+    assert abs(g["mean_prob"].sum() - 1.0) < 1e-5
+    assert abs(g["mean_count"].sum() - k) < 1e-5
+    # a transposed or mis-scaled term would break this: doubling one expert's count moves the loss
+    # by exactly mean_prob[e] * count[e] / (S * E)
+    cnt2 = r["expert_count"].copy(); cnt2[5] *= 2
+    g2 = oracle.gate_loss(c, r["probs"], cnt2)
+    assert abs((g2["loss"] - g["loss"]) - g["mean_prob"][5] * r["expert_count"][5] / (S * E)) < 1e-7
