@@ -12,6 +12,9 @@ namespace kleos_amd {
 typedef __bf16 bf16_t;
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16_t;
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -20,6 +23,7 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 constexpr int kWave = 64;
 
 __device__ __forceinline__ float elem_to_float(bf16_t v) { return static_cast<float>(v); }
+__device__ __forceinline__ float elem_to_float(f16_t v) { return static_cast<float>(v); }
 __device__ __forceinline__ float elem_to_float(float v) { return v; }
 
 // fp32 -> Element, round to nearest even (cutlass::NumericConverter in the reference).
@@ -29,6 +33,26 @@ template <>
 __device__ __forceinline__ float float_to_elem<float>(float v) { return v; }
 template <>
 __device__ __forceinline__ bf16_t float_to_elem<bf16_t>(float v) { return static_cast<bf16_t>(v); }
+template <>
+__device__ __forceinline__ f16_t float_to_elem<f16_t>(float v) { return static_cast<f16_t>(v); }
+
+// The two 16-bit Elements share every kernel; what differs is the vector types and the matrix
+// instructions.
+template <typename E> struct Elem16;
+template <> struct Elem16<bf16_t> {
+    typedef bf16x8 vec8;
+    typedef bf16x4 vec4;
+    static __device__ __forceinline__ f32x16 mfma32(vec8 a, vec8 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    }
+};
+template <> struct Elem16<f16_t> {
+    typedef f16x8 vec8;
+    typedef f16x4 vec4;
+    static __device__ __forceinline__ f32x16 mfma32(vec8 a, vec8 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+};
 
 __device__ __forceinline__ u32x4 load16(const void* p) { return *reinterpret_cast<const u32x4*>(p); }
 __device__ __forceinline__ void store16(void* p, u32x4 v) { *reinterpret_cast<u32x4*>(p) = v; }
@@ -49,6 +73,10 @@ __device__ __forceinline__ float activate(float v) {
 __device__ __forceinline__ f32x4 mma16_step(u32x4 a, u32x4 b, f32x4 acc, bf16_t) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a),
                                                    __builtin_bit_cast(bf16x8, b), acc, 0, 0, 0);
+}
+__device__ __forceinline__ f32x4 mma16_step(u32x4 a, u32x4 b, f32x4 acc, f16_t) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a),
+                                                  __builtin_bit_cast(f16x8, b), acc, 0, 0, 0);
 }
 __device__ __forceinline__ f32x4 mma16_step(u32x4 a, u32x4 b, f32x4 acc, float) {
     f32x4 fa = __builtin_bit_cast(f32x4, a), fb = __builtin_bit_cast(f32x4, b);

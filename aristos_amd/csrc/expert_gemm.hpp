@@ -12,7 +12,7 @@
 namespace kleos_amd {
 
 // ------------------------------------------------------------------------------------------------
-// bf16, matrix cores. WAVES_M x WAVES_N wavefronts over a BM x BN tile.
+// 16-bit Elements (bf16, fp16), matrix cores. WAVES_M x WAVES_N wavefronts over a BM x BN tile.
 //
 // K is walked in slices of BK through a ring of LDS stages that the wavefronts fill with direct
 // global->LDS loads (global_load_lds_dwordx4: each lane names a 16-byte global source, the 64 lanes
@@ -50,21 +50,27 @@ __device__ __forceinline__ void wait_vmcnt() {
     __builtin_amdgcn_s_waitcnt(0x0f70 | (N & 15) | ((N >> 4) << 14));
 }
 
+// A 16-bit Element seen only as storage: addresses are computed in units of it, values are
+// interpreted by the Element type the tile is instantiated with.
+typedef uint16_t elem16_t;
+
 // What one output tile needs, in scalar form (identical in every lane).
 struct GemmTileArgs {
-    const bf16_t* a_base;          // A rows (gathered through a_row_index when it is not null)
+    const elem16_t* a_base;        // A rows (gathered through a_row_index when it is not null)
     const int32_t* a_row_index;
     uint32_t a_rows;               // rows behind a_base: gathered indices are clamped below it
-    const bf16_t* b_base;          // first of the tile's weight rows
-    const bf16_t* bias;            // first of the tile's bias entries
-    bf16_t* c_base;                // output element (row 0, column 0) of the tile
+    const elem16_t* b_base;        // first of the tile's weight rows
+    const elem16_t* bias;          // first of the tile's bias entries
+    elem16_t* c_base;              // output element (row 0, column 0) of the tile
     uint32_t lda, ldb, ldc, K;
     uint32_t m_valid, n_valid;     // rows / columns of the tile that exist
     uint32_t act;                  // 0 relu, 1 erf-gelu, 2 identity
 };
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES>
-struct GemmBf16 {
+template <typename E, int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES>
+struct Gemm16 {
+    typedef typename Elem16<E>::vec8 vec8;
+    typedef typename Elem16<E>::vec4 vec4;
     static constexpr int kWaves = WAVES_M * WAVES_N;
     static constexpr int kThreads = kWaves * kWave;
     static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;     // wavefront tile
@@ -96,9 +102,9 @@ struct GemmBf16 {
     }
 
     struct Tile {
-        const bf16_t* pa[LA];
-        const bf16_t* pb[LB];
-        bf16_t* c_base;
+        const elem16_t* pa[LA];
+        const elem16_t* pb[LB];
+        elem16_t* c_base;
         uint32_t ldc, m_valid, n_valid, k_tiles, act;
         int stage0;                 // stage of K slice 0; slice kt uses (stage0 + kt) % STAGES
         int bias_slot;              // which of the two LDS bias slots holds this tile's bias
@@ -207,12 +213,12 @@ struct GemmBf16 {
             const char* st = smem + stage_of(t, kt) * kStage;
             // The operand fragments of K step ks+1 are read from LDS while the matrix core works
             // on step ks.
-            bf16x8 fw[2][TN], fx[2][TM];
+            vec8 fw[2][TN], fx[2][TM];
             auto read_fragments = [&](int ks) {
 #pragma unroll
-                for (int ni = 0; ni < TN; ++ni) fw[ks & 1][ni] = __builtin_bit_cast(bf16x8, load16(st + (base_w ^ (ks << 5)) + ni * 32 * kRowBytes));
+                for (int ni = 0; ni < TN; ++ni) fw[ks & 1][ni] = __builtin_bit_cast(vec8, load16(st + (base_w ^ (ks << 5)) + ni * 32 * kRowBytes));
 #pragma unroll
-                for (int mi = 0; mi < TM; ++mi) fx[ks & 1][mi] = __builtin_bit_cast(bf16x8, load16(st + (base_x ^ (ks << 5)) + mi * 32 * kRowBytes));
+                for (int mi = 0; mi < TM; ++mi) fx[ks & 1][mi] = __builtin_bit_cast(vec8, load16(st + (base_x ^ (ks << 5)) + mi * 32 * kRowBytes));
             };
             read_fragments(0);
 #pragma unroll
@@ -224,7 +230,7 @@ struct GemmBf16 {
                 for (int ni = 0; ni < TN; ++ni)
 #pragma unroll
                     for (int mi = 0; mi < TM; ++mi)
-                        acc[ni][mi] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fw[ks & 1][ni], fx[ks & 1][mi], acc[ni][mi], 0, 0, 0);
+                        acc[ni][mi] = Elem16<E>::mfma32(fw[ks & 1][ni], fx[ks & 1][mi], acc[ni][mi]);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
@@ -260,12 +266,12 @@ struct GemmBf16 {
                     const int ni = pn * 2 + nl;
 #pragma unroll
                     for (int q = 0; q < 4; ++q) {
-                        const bf16x4 b4 = *reinterpret_cast<const bf16x4*>(bias_lane + (ni * 32 + 8 * q) * 2);
-                        bf16x4 o;
+                        const vec4 b4 = *reinterpret_cast<const vec4*>(bias_lane + (ni * 32 + 8 * q) * 2);
+                        vec4 o;
 #pragma unroll
                         for (int j = 0; j < 4; ++j)
-                            o[j] = static_cast<bf16_t>(activate<ACT>(acc[ni][mi][4 * q + j] + float(b4[j])));
-                        *reinterpret_cast<bf16x4*>(stg + fr_row * 128 + (((nl * 4 + q) ^ ((fr_row >> 1) & 7)) << 4) + fr_half * 8) = o;
+                            o[j] = static_cast<E>(activate<ACT>(acc[ni][mi][4 * q + j] + float(b4[j])));
+                        *reinterpret_cast<vec4*>(stg + fr_row * 128 + (((nl * 4 + q) ^ ((fr_row >> 1) & 7)) << 4) + fr_half * 8) = o;
                     }
                 }
                 // the same wavefront wrote and reads the region: LDS operations of one wavefront

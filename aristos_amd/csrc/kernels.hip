@@ -31,20 +31,22 @@ constexpr int kXcds = 8;
 // (two per SIMD), K slices of 64 (whole 128-byte lines of every row) through two 64 KB stages.
 // (Measured against it on MI355X, none faster: K slices of 32 through four stages, all loads of a
 // slice issued at its first K step, 2 x 2 wavefronts of 128 x 128 with the accumulators in AGPRs.)
-using GemmCfg = GemmBf16<256, 256, 2, 4, 64, 2>;
+template <typename E>
+using GemmCfg = Gemm16<E, 256, 256, 2, 4, 64, 2>;
 constexpr int kBM = 256, kBN = 256;
-constexpr int kGemmThreads = GemmCfg::kThreads;
+constexpr int kGemmThreads = GemmCfg<bf16_t>::kThreads;
 
 // Tile shape and workgroup size of the expert projections per Element type. The workgroup size is
 // also that of the persistent kernel, whose other phases run on groups of its wavefronts.
 template <typename T> struct TileShape;
 template <> struct TileShape<bf16_t> { static constexpr int BM = kBM, BN = kBN, kThreads = kGemmThreads, kPerCu = 1; };
+template <> struct TileShape<f16_t> : TileShape<bf16_t> {};
 template <> struct TileShape<float> { static constexpr int BM = kF32Tile, BN = kF32Tile, kThreads = 256, kPerCu = 1; };
 constexpr int kPhaseThreads = 256;   // gate, slot and combine kernels of the phased mode
 
 template <typename T>
 constexpr int gemm_smem_bytes() {
-    if constexpr (sizeof(T) == 2) return GemmCfg::kSmemBytes;
+    if constexpr (sizeof(T) == 2) return GemmCfg<T>::kSmemBytes;
     else return gemm_f32_smem_bytes();
 }
 constexpr int kPhasedGemmHeader = 128;
@@ -256,11 +258,13 @@ __device__ __forceinline__ void expert_loop(const LayerParams& p, char* smem, ui
     };
 
     if constexpr (sizeof(T) == 2) {
-        using G = GemmCfg;
+        using G = GemmCfg<T>;
         auto args_of = [&](const Task& t) {
             const TileOperands<T> o = tile_operands<T>(p, t);
             GemmTileArgs g;
-            g.a_base = o.a; g.a_row_index = o.idx; g.a_rows = p.S; g.b_base = o.w; g.bias = o.bias; g.c_base = o.c;
+            g.a_base = reinterpret_cast<const elem16_t*>(o.a); g.a_row_index = o.idx; g.a_rows = p.S;
+            g.b_base = reinterpret_cast<const elem16_t*>(o.w); g.bias = reinterpret_cast<const elem16_t*>(o.bias);
+            g.c_base = reinterpret_cast<elem16_t*>(o.c);
             g.lda = o.lda; g.ldb = o.K; g.ldc = o.ldc; g.K = o.K; g.m_valid = o.m_valid; g.n_valid = o.n_valid;
             g.act = o.act;
             return g;
@@ -541,6 +545,16 @@ int gate_groups(uint32_t E) {
     return 16;
 }
 
+// Calls go(Element{}) for the Element type of a torch_dtype value (kleos_amd.h: 0 fp32, 2 bf16, 3 fp16).
+template <typename F>
+hipError_t dispatch_dtype(int dtype, F&& go) {
+    switch (dtype) {
+        case 2: return go(bf16_t{});
+        case 3: return go(f16_t{});
+        default: return go(float{});
+    }
+}
+
 template <typename F>
 hipError_t dispatch_groups(uint32_t E, F&& f) {
     switch (gate_groups(E)) {
@@ -585,7 +599,7 @@ hipError_t launch_gate(const LayerParams& p, int dtype, hipStream_t s) {
                                smem, s, p);
             return hipGetLastError();
         };
-        return dtype == 2 ? go(bf16_t{}) : go(float{});
+        return dispatch_dtype(dtype, go);
     });
 }
 
@@ -622,14 +636,15 @@ hipError_t launch_expert_gemm(const LayerParams& p, int dtype, int kind, int num
         hipLaunchKernelGGL(kernel, dim3(grid), dim3(TileShape<T>::kThreads), smem, s, p, uint32_t(kind), tiles_m, tiles_n);
         return hipGetLastError();
     };
-    return dtype == 2 ? go(bf16_t{}) : go(float{});
+    return dispatch_dtype(dtype, go);
 }
 
 hipError_t launch_combine(const LayerParams& p, int dtype, hipStream_t s) {
     const uint32_t grid = ceil_div_u32(p.S, 4);
-    if (dtype == 2) hipLaunchKernelGGL((combine_kernel<bf16_t>), dim3(grid), dim3(kPhaseThreads), 0, s, p);
-    else hipLaunchKernelGGL((combine_kernel<float>), dim3(grid), dim3(kPhaseThreads), 0, s, p);
-    return hipGetLastError();
+    return dispatch_dtype(dtype, [&](auto tag) {
+        hipLaunchKernelGGL((combine_kernel<decltype(tag)>), dim3(grid), dim3(kPhaseThreads), 0, s, p);
+        return hipGetLastError();
+    });
 }
 
 hipError_t plan_fused(const LayerParams& p, int dtype, int num_cus, FusedPlan* plan) {
@@ -661,7 +676,7 @@ hipError_t plan_fused(const LayerParams& p, int dtype, int num_cus, FusedPlan* p
             plan->threads = TileShape<T>::kThreads;
             return hipSuccess;
         };
-        return dtype == 2 ? go(bf16_t{}) : go(float{});
+        return dispatch_dtype(dtype, go);
     });
 }
 

@@ -97,7 +97,9 @@ def scaled(workload: Workload, **overrides) -> Workload:
 
 def _torch_dtype(derived: DerivedConfig):
     import torch
-    return torch.float32 if derived.elem_bytes == 4 else torch.bfloat16
+    if derived.elem_bytes == 4:
+        return torch.float32
+    return torch.float16 if derived.keys.torch_dtype == 3 else torch.bfloat16
 
 
 def make_inputs(workload: Workload, seed: int = 0, device: str = "cuda", portable: bool = False):

@@ -70,7 +70,7 @@ typedef struct kleos_config {
     uint32_t cap_rows;          /* min(pEC, S): row stride of every per-expert buffer. An expert
                                  * never holds more than S tokens, so without token dropping
                                  * (EC = S*cf*k) the arenas are sized by S instead.              */
-    uint32_t elem_bytes;        /* sizeof(Element): 4 (fp32) or 2 (bf16)                         */
+    uint32_t elem_bytes;        /* sizeof(Element): 4 (fp32) or 2 (bf16, fp16)                   */
     /* Element offsets into the packed input buffer iP (csrc/include/kleos/moe/moe.cuh:92-96,
      * csrc/main.cu:23-28) and the packed output buffer oP (moe.cuh:97-98). */
     uint64_t off_x, off_gate_w, off_w_up, off_w_down, off_b_up, off_b_down, in_elems;
@@ -86,7 +86,7 @@ int kleos_config_parse_file(const char* path, kleos_config_t* cfg);
 void kleos_config_defaults(kleos_config_t* cfg);
 /* Validate the keys and fill the derived fields. Enforces the reference's static_asserts
  * (csrc/include/kleos/bootstrap.cuh:542-545; types.cuh:479,496-497): S % 128 == 0, I % 64 == 0,
- * H % 64 == 0, k <= E, E <= 65535, capacity_factor >= 1. tf32 and fp16 yield KLEOS_EUNSUPPORTED. */
+ * H % 64 == 0, k <= E, E <= 65535, capacity_factor >= 1. tf32 yields KLEOS_EUNSUPPORTED. */
 int kleos_config_derive(kleos_config_t* cfg);
 
 /* ---- lifecycle ------------------------------------------------------------------------------ */

@@ -66,20 +66,69 @@ float moe_ref_bf16_bits_to_f32(uint16_t b) {
 }
 float moe_ref_round_bf16(float v) { return moe_ref_bf16_bits_to_f32(moe_ref_f32_to_bf16_bits(v)); }
 
-static inline float to_elem(float v, uint32_t dtype) { return dtype == 2 ? moe_ref_round_bf16(v) : v; }
+/* IEEE binary16 by integer arithmetic: round to nearest, ties to even; overflow to infinity,
+ * gradual underflow to subnormals (what cutlass::NumericConverter<half_t, float> does). */
+uint16_t moe_ref_f32_to_f16_bits(float v) {
+    uint32_t u;
+    memcpy(&u, &v, 4);
+    const uint16_t sign = (uint16_t)((u >> 16) & 0x8000u);
+    const uint32_t a = u & 0x7fffffffu;
+    if (a > 0x7f800000u) return (uint16_t)(sign | 0x7e00u);          /* NaN */
+    if (a >= 0x47800000u) return (uint16_t)(sign | 0x7c00u);         /* >= 65536 (and inf): infinity */
+    if (a < 0x33000000u) return sign;                                /* < 2^-25: zero */
+    const int exp = (int)(a >> 23) - 127;
+    uint32_t mant = (a & 0x007fffffu) | 0x00800000u;                 /* 24-bit significand */
+    int shift;                                                       /* bits dropped from it */
+    uint32_t base;                                                   /* half bits before the mantissa is added */
+    if (exp < -14) { shift = 13 + (-14 - exp); base = 0; }           /* subnormal half */
+    else { shift = 13; base = (uint32_t)(exp + 15 - 1) << 10; }      /* implicit bit carries into the exponent */
+    const uint32_t kept = mant >> shift;
+    const uint32_t rem = mant & ((1u << shift) - 1u);
+    const uint32_t half = 1u << (shift - 1);
+    uint32_t h = base + kept;
+    if (rem > half || (rem == half && (kept & 1u))) ++h;             /* may carry up to infinity: correct */
+    return (uint16_t)(sign | h);
+}
+float moe_ref_f16_bits_to_f32(uint16_t b) {
+    const uint32_t sign = (uint32_t)(b & 0x8000u) << 16;
+    const uint32_t exp = (b >> 10) & 0x1fu, mant = b & 0x3ffu;
+    uint32_t u;
+    if (exp == 0x1fu) u = sign | 0x7f800000u | (mant << 13);
+    else if (exp != 0) u = sign | ((exp + 112u) << 23) | (mant << 13);
+    else if (mant == 0) u = sign;
+    else {
+        /* subnormal: value = mant * 2^-24 */
+        float v = (float)mant * 5.9604644775390625e-08f;
+        memcpy(&u, &v, 4);
+        u |= sign;
+    }
+    float v;
+    memcpy(&v, &u, 4);
+    return v;
+}
+float moe_ref_round_f16(float v) { return moe_ref_f16_bits_to_f32(moe_ref_f32_to_f16_bits(v)); }
+
+static inline float to_elem(float v, uint32_t dtype) {
+    return dtype == 2 ? moe_ref_round_bf16(v) : dtype == 3 ? moe_ref_round_f16(v) : v;
+}
 
 /* Packed-buffer element i as fp32. */
 static inline float load_elem(const void* p, size_t i, uint32_t dtype) {
-    return dtype == 2 ? moe_ref_bf16_bits_to_f32(((const uint16_t*)p)[i]) : ((const float*)p)[i];
+    return dtype == 2 ? moe_ref_bf16_bits_to_f32(((const uint16_t*)p)[i])
+         : dtype == 3 ? moe_ref_f16_bits_to_f32(((const uint16_t*)p)[i]) : ((const float*)p)[i];
 }
 static inline void store_elem(void* p, size_t i, float v, uint32_t dtype) {
     if (dtype == 2) ((uint16_t*)p)[i] = moe_ref_f32_to_bf16_bits(v);
+    else if (dtype == 3) ((uint16_t*)p)[i] = moe_ref_f32_to_f16_bits(v);
     else ((float*)p)[i] = v;
 }
 static void load_elems(const void* p, size_t off, size_t n, uint32_t dtype, float* dst) {
     if (dtype == 2) {
         const uint16_t* s = (const uint16_t*)p + off;
         for (size_t i = 0; i < n; ++i) dst[i] = moe_ref_bf16_bits_to_f32(s[i]);
+    } else if (dtype == 3) {
+        const uint16_t* s = (const uint16_t*)p + off;
+        for (size_t i = 0; i < n; ++i) dst[i] = moe_ref_f16_bits_to_f32(s[i]);
     } else {
         memcpy(dst, (const float*)p + off, n * sizeof(float));
     }
@@ -116,7 +165,7 @@ int moe_ref_threads(void) {
 int moe_ref_derive(moe_ref_cfg* c) {
     if (!c || !c->S || !c->H || !c->I || !c->E || !c->k || c->k > c->E) return -1;
     if (c->S % 128 || c->H % 64 || c->I % 64 || !(c->capacity_factor >= 1.0)) return -1;
-    if (c->dtype != 0 && c->dtype != 2) return -1;
+    if (c->dtype != 0 && c->dtype != 2 && c->dtype != 3) return -1;
     c->PX = (c->E + 63u) / 64u * 64u;                                   /* types.cuh:481 */
     double base = c->drop_tokens ? (double)((c->S + c->E - 1u) / c->E) : (double)c->S;
     c->EC = (uint32_t)ceil(base * c->capacity_factor * (double)c->k - 1e-9); /* types.cuh:498-499 */

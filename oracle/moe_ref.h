@@ -19,7 +19,7 @@ typedef struct moe_ref_cfg {
     double capacity_factor;
     uint32_t drop_tokens;   /* 0 | 1 */
     uint32_t hidden_act;    /* 0 relu | 1 erf-gelu */
-    uint32_t dtype;         /* 0 fp32 | 2 bf16 (Element) */
+    uint32_t dtype;         /* 0 fp32 | 2 bf16 | 3 fp16 (Element) */
     /* derived by moe_ref_derive */
     uint32_t PX, EC, pEC, cap_rows;
 } moe_ref_cfg;
@@ -31,6 +31,9 @@ int moe_ref_derive(moe_ref_cfg* c);
 float moe_ref_round_bf16(float v);
 uint16_t moe_ref_f32_to_bf16_bits(float v);
 float moe_ref_bf16_bits_to_f32(uint16_t b);
+float moe_ref_round_f16(float v);
+uint16_t moe_ref_f32_to_f16_bits(float v);
+float moe_ref_f16_bits_to_f32(uint16_t b);
 
 /* logits[t,e] = sum_h x[t,h] * wg[e,h], fp32 accumulation. x [S,H], wg [E,H], logits [S,E]. */
 void moe_ref_gate_logits(uint32_t S, uint32_t H, uint32_t E, const float* x, const float* wg,

@@ -53,6 +53,12 @@ def lib() -> C.CDLL:
         h.moe_ref_threads.restype = C.c_int
         h.moe_ref_round_bf16.restype = C.c_float
         h.moe_ref_round_bf16.argtypes = [C.c_float]
+        h.moe_ref_round_f16.restype = C.c_float
+        h.moe_ref_round_f16.argtypes = [C.c_float]
+        h.moe_ref_f32_to_f16_bits.restype = C.c_uint16
+        h.moe_ref_f32_to_f16_bits.argtypes = [C.c_float]
+        h.moe_ref_f16_bits_to_f32.restype = C.c_float
+        h.moe_ref_f16_bits_to_f32.argtypes = [C.c_uint16]
         h.moe_ref_gate_logits.restype = None
         h.moe_ref_gate_logits.argtypes = [C.c_uint32, C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p]
         h.moe_ref_softmax.restype = None
@@ -99,7 +105,7 @@ def out_elems(c: RefCfg) -> int:
 
 
 def elem_np_dtype(c: RefCfg):
-    return np.uint16 if c.dtype == 2 else np.float32
+    return np.uint16 if c.dtype in (2, 3) else np.float32
 
 
 def bf16_bits_to_f32(a: np.ndarray) -> np.ndarray:
@@ -112,8 +118,21 @@ def f32_to_bf16_bits(a: np.ndarray) -> np.ndarray:
     return (rounded >> 16).astype(np.uint16)
 
 
+def f32_to_elem_bits(a: np.ndarray, c: RefCfg) -> np.ndarray:
+    """fp32 values -> the packed Element representation of the configuration."""
+    if c.dtype == 2:
+        return f32_to_bf16_bits(a)
+    if c.dtype == 3:
+        return np.ascontiguousarray(a, dtype=np.float32).astype(np.float16).view(np.uint16)
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
 def elems_to_f32(a: np.ndarray, c: RefCfg) -> np.ndarray:
-    return bf16_bits_to_f32(a) if c.dtype == 2 else a.astype(np.float32)
+    if c.dtype == 2:
+        return bf16_bits_to_f32(a)
+    if c.dtype == 3:
+        return np.ascontiguousarray(a).view(np.float16).astype(np.float32)
+    return a.astype(np.float32)
 
 
 def forward(c: RefCfg, iP: np.ndarray, logits: np.ndarray | None = None,

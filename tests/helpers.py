@@ -21,9 +21,7 @@ def pack_inputs(c, x, wg, w_up, w_down, b_up=None, b_down=None) -> np.ndarray:
     o += E * I
     if b_down is not None:
         buf[o:o + E * H] = np.asarray(b_down, np.float32).ravel()
-    if c.dtype == 2:
-        return moe_ref.f32_to_bf16_bits(buf)
-    return buf
+    return moe_ref.f32_to_elem_bits(buf, c)
 
 
 def unpack_inputs(c, iP: np.ndarray):
@@ -59,4 +57,7 @@ def random_layer(c, seed=0, x_std=1.0, w_std=0.02, bias_std=0.0):
     if c.dtype == 2:
         from np_restatement import round_bf16
         x, wg, w_up, w_down, b_up, b_down = (round_bf16(a) for a in (x, wg, w_up, w_down, b_up, b_down))
+    if c.dtype == 3:
+        x, wg, w_up, w_down, b_up, b_down = (a.astype(np.float16).astype(np.float32)
+                                             for a in (x, wg, w_up, w_down, b_up, b_down))
     return x, wg, w_up, w_down, b_up, b_down

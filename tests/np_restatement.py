@@ -28,8 +28,11 @@ def round_bf16(a: np.ndarray) -> np.ndarray:
     return (r & 0xFFFFFFFF).astype(np.uint32).view(np.float32).reshape(a.shape)
 
 
-def to_elem(a, bf16: bool):
+def to_elem(a, bf16):
+    """bf16: True / "bf16" -> bfloat16, "f16" -> IEEE half (numpy's conversion), False -> fp32."""
     a = np.asarray(a, dtype=np.float32)
+    if bf16 == "f16":
+        return a.astype(np.float16).astype(np.float32)
     return round_bf16(a) if bf16 else a
 
 
@@ -70,9 +73,11 @@ def gelu_erf(v):
     return 0.5 * v * (1.0 + erf(v / math.sqrt(2.0)))
 
 
-def forward(x, wg, w_up, w_down, b_up, b_down, k, cf=1.0, drop=1, act=0, bf16=True, logits=None):
+def forward(x, wg, w_up, w_down, b_up, b_down, k, cf=1.0, drop=1, act=0, bf16=True, logits=None, elem=None):
     """x [S,H], wg [E,H], w_up [E,I,H], w_down [E,H,I], b_up [E,I], b_down [E,H]; all fp32 arrays
     holding Element-representable values. Returns a dict like the C oracle's."""
+    if elem is not None:
+        bf16 = elem
     S, H = x.shape
     E = wg.shape[0]
     PX, EC, pEC, cap_rows = derive(S, E, k, cf, drop)

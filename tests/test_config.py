@@ -63,7 +63,6 @@ def test_integer_capacity_factor_matches_reference_formula():
     ({"capacity_factor": 0.5}, _capi.KLEOS_EINVAL, "capacity_factor"),
     ({"hidden_act": 2}, _capi.KLEOS_EINVAL, "hidden_act"),
     ({"drop_tokens": 2}, _capi.KLEOS_EINVAL, "drop_tokens"),
-    ({"torch_dtype": 3}, _capi.KLEOS_EUNSUPPORTED, "fp16"),
 ])
 def test_invalid_configs_are_rejected_with_a_message(override, code, needle):
     with pytest.raises(ka.KleosError) as ei:

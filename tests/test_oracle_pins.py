@@ -323,3 +323,36 @@ def test_gate_loss_vs_numpy_and_invariants(oracle):
     cnt2 = r["expert_count"].copy(); cnt2[5] *= 2
     g2 = oracle.gate_loss(c, r["probs"], cnt2)
     assert abs((g2["loss"] - g["loss"]) - g["mean_prob"][5] * r["expert_count"][5] / (S * E)) < 1e-7
+
+
+# ------------------------------------------------------------------ fp16 Element
+def test_f16_round_matches_numpy(oracle):
+    """The oracle's integer-arithmetic binary16 conversion against numpy's float16 (an independent
+    implementation): random values over the whole range, exact ties, subnormals, overflow."""
+    rng = np.random.default_rng(5)
+    vals = np.concatenate([
+        rng.standard_normal(4000).astype(np.float32) * np.float32(10.0) ** rng.integers(-9, 6, 4000).astype(np.float32),
+        np.array([0.0, -0.0, 1.0, 65504.0, 65519.9, 65520.0, 65536.0, 1e6, -1e6, 2.0**-24, 2.0**-25, 1.5 * 2.0**-25,
+                  2.0**-26, 6.1e-5, 6.097555e-05, 1.0 + 2.0**-11, 1.0 + 3 * 2.0**-11, 1.0 + 2.0**-11 + 2.0**-20],
+                 dtype=np.float32),
+    ])
+    lib = oracle.lib()
+    got = np.array([lib.moe_ref_f32_to_f16_bits(float(v)) for v in vals], dtype=np.uint16)
+    with np.errstate(over="ignore"):
+        want = vals.astype(np.float16).view(np.uint16)
+    np.testing.assert_array_equal(got, want)
+    back = np.array([lib.moe_ref_f16_bits_to_f32(int(b)) for b in range(0, 0x7c00, 7)], dtype=np.float32)
+    np.testing.assert_array_equal(back, np.arange(0, 0x7c00, 7, dtype=np.uint16).view(np.float16).astype(np.float32))
+
+
+def test_layer_fp16_vs_numpy_restatement(oracle):
+    """Whole layer with fp16 Elements against the independent restatement (which rounds with
+    numpy's float16)."""
+    c = oracle.make_cfg(S=128, H=64, I=128, E=8, k=2, dtype=3)
+    x, wg, w_up, w_down, b_up, b_down = random_layer(c, seed=3, w_std=0.1, bias_std=0.05)
+    iP = pack_inputs(c, x, wg, w_up, w_down, b_up, b_down)
+    got = oracle.forward(c, iP)
+    ref = npr.forward(x, wg, w_up, w_down, b_up, b_down, k=2, elem="f16")
+    np.testing.assert_array_equal(got["topk_expert"], ref["topk_expert"])
+    np.testing.assert_array_equal(got["topk_slot"], ref["topk_slot"])
+    assert rel_fro(got["moe_out"], ref["moe_out"]) < 2e-3
