@@ -8,6 +8,8 @@ summation order, so it is checked "given the same fp32 logits"):
   3. oracle outputs computed from the GPU's logits vs GPU outputs: relative Frobenius error
      <= 1e-2 for bf16, <= 1e-5 for fp32 (the tolerances the task states).
 """
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -394,3 +396,21 @@ def test_gate_loss_needs_training_mode():
             ka.moe.gate_loss(d.E)
     finally:
         ka.finalize()
+
+
+# ------------------------------------------------------------------ the reference's driver, on this library
+def test_cpp_driver_prints_the_reference_line(tmp_path):
+    """csrc/kleos_main is the equivalent of the reference's runOS() (csrc/main.cu:13-73): it reads a
+    kleos_config.json, fills the packed buffers on the host, runs forwardHostBench<32,32> through
+    kleos.hpp and prints `epRank: 0 took X ms`."""
+    import re
+    import subprocess
+    from aristos_amd import build
+    if not os.path.exists(build.DRIVER_PATH):
+        pytest.skip("the C++ driver is not built")
+    cfg = tmp_path / "kleos_config.json"
+    cfg.write_text(_keys(1024, 256, 256, 16, 2).to_json_text())
+    r = subprocess.run([build.DRIVER_PATH, str(cfg)], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stderr
+    m = re.search(r"epRank: 0 took ([0-9.]+)\s*ms", r.stdout)
+    assert m and float(m.group(1)) > 0, r.stdout
