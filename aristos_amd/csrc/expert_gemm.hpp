@@ -67,6 +67,80 @@ struct GemmTileArgs {
     uint32_t act;                  // 0 relu, 1 erf-gelu, 2 identity
 };
 
+// Where a tile's results go.
+struct TileOut {
+    elem16_t* c_base;              // output element (row 0, column 0) of the tile
+    uint32_t ldc, m_valid, n_valid, act;
+};
+
+// The lane's thread index as a value the optimiser cannot trace back to threadIdx: whatever a
+// phase derives from it is computed when the phase starts and dies when it ends, instead of
+// being shared with the main loop and kept (or spilled) across it.
+__device__ __forceinline__ uint32_t local_tid() {
+    uint32_t t = threadIdx.x;
+    asm volatile("" : "+v"(t));
+    return t;
+}
+
+// Epilogue of a WAVES_M x WAVES_N wavefront grid whose wavefronts each hold a WM x WN block of the
+// C^T accumulators: acc[ni][mi][v] is output column n = wn*WN + ni*32 + 8*(v/4) + 4*(lane/32) + v%4
+// of output row m = wm*WM + mi*32 + lane%32, i.e. a lane owns 4 consecutive columns of 16 rows per
+// 32x32 block. Bias, activation and the rounding to Element happen in registers; the wavefront
+// then transposes 32-row x 64-column panels through a private LDS region of 4 KB at
+// stage_mem + wave * 4096 (rows of 128 bytes, 16-byte chunk c of row r at position
+// c ^ ((r >> 1) & 7)) so that the global stores are 16 bytes per lane and cover whole 128-byte
+// lines of the output rows. The bias comes from LDS (bias_mem: the tile's BN entries): the epilogue
+// issues no global load, so nothing in it ever waits for the stores it has in flight.
+constexpr int kEpiloguePanelRows = 32;
+template <typename E, int WM, int WN, int WAVES_N, int ACT>
+__device__ __forceinline__ void epilogue16_act(const TileOut& t, f32x16 (&acc)[WN / 32][WM / 32], char* stage_mem,
+                                               const char* bias_mem) {
+    typedef typename Elem16<E>::vec4 vec4;
+    constexpr int TM = WM / 32, kPanelRows = kEpiloguePanelRows;
+    const uint32_t tid = local_tid();
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+    const int fr_row = lane & 31, fr_half = lane >> 5;
+    char* stg = stage_mem + wave * (kPanelRows * 128);
+    const char* bias_lane = bias_mem + (wn * WN + 4 * fr_half) * 2;
+#pragma unroll
+    for (int mi = 0; mi < TM; ++mi) {
+#pragma unroll
+        for (int pn = 0; pn < WN / 64; ++pn) {
+#pragma unroll
+            for (int nl = 0; nl < 2; ++nl) {
+                const int ni = pn * 2 + nl;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const vec4 b4 = *reinterpret_cast<const vec4*>(bias_lane + (ni * 32 + 8 * q) * 2);
+                    vec4 o;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        o[j] = static_cast<E>(activate<ACT>(acc[ni][mi][4 * q + j] + float(b4[j])));
+                    *reinterpret_cast<vec4*>(stg + fr_row * 128 + (((nl * 4 + q) ^ ((fr_row >> 1) & 7)) << 4) + fr_half * 8) = o;
+                }
+            }
+            // the same wavefront wrote and reads the region: LDS operations of one wavefront
+            // complete in order
+#pragma unroll
+            for (int it = 0; it < kPanelRows * 8 / kWave; ++it) {
+                const int id = it * kWave + lane;
+                const int r = id >> 3, c = id & 7;
+                const u32x4 v = load16(stg + r * 128 + ((c ^ ((r >> 1) & 7)) << 4));
+                const uint32_t m = wm * WM + mi * 32 + r, n = wn * WN + pn * 64 + c * 8;
+                if (m < t.m_valid && n < t.n_valid) store16(t.c_base + size_t(m) * t.ldc + n, v);
+            }
+        }
+    }
+}
+template <typename E, int WM, int WN, int WAVES_N>
+__device__ __forceinline__ void epilogue16(const TileOut& t, f32x16 (&acc)[WN / 32][WM / 32], char* stage_mem,
+                                           const char* bias_mem) {
+    if (t.act == 0) epilogue16_act<E, WM, WN, WAVES_N, 0>(t, acc, stage_mem, bias_mem);
+    else if (t.act == 1) epilogue16_act<E, WM, WN, WAVES_N, 1>(t, acc, stage_mem, bias_mem);
+    else epilogue16_act<E, WM, WN, WAVES_N, 2>(t, acc, stage_mem, bias_mem);
+}
+
 template <typename E, int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES>
 struct Gemm16 {
     typedef typename Elem16<E>::vec8 vec8;
@@ -86,7 +160,7 @@ struct Gemm16 {
     static constexpr int LA = BM / (kRowsPerLoad * kWaves), LB = BN / (kRowsPerLoad * kWaves);
     static constexpr int kLoadsPerSlice = LA + LB;                 // per wavefront
     static constexpr int kSteps = BK / 16;                         // matrix instructions consume 16 values of K
-    static constexpr int kPanelRows = 32;                          // epilogue staging: 32 rows x 64 columns per wavefront
+    static constexpr int kPanelRows = kEpiloguePanelRows;          // epilogue staging: 32 rows x 64 columns per wavefront
     static constexpr int kIssueSteps = kSteps;                     // K steps over which the next slice's loads are issued
     static_assert(BK == 32 || BK == 64);
     static_assert(STAGES >= 2 && STAGES <= 4);
@@ -109,15 +183,6 @@ struct Gemm16 {
         int stage0;                 // stage of K slice 0; slice kt uses (stage0 + kt) % STAGES
         int bias_slot;              // which of the two LDS bias slots holds this tile's bias
     };
-
-    // The lane's thread index as a value the optimiser cannot trace back to threadIdx: whatever a
-    // phase derives from it is computed when the phase starts and dies when it ends, instead of
-    // being shared with the main loop and kept (or spilled) across it.
-    static __device__ __forceinline__ uint32_t local_tid() {
-        uint32_t t = threadIdx.x;
-        asm volatile("" : "+v"(t));
-        return t;
-    }
 
     typedef f32x16 Acc[TN][TM];
 
@@ -241,60 +306,10 @@ struct Gemm16 {
     // The stage the next tile's first slice must go to.
     static __device__ __forceinline__ int next_stage0(const Tile& t) { return (t.stage0 + t.k_tiles) % STAGES; }
 
-    template <int ACT>
-    static __device__ __forceinline__ void finish_act(const Tile& t, Acc& acc, char* stage_mem, const char* bias_mem) {
-        // acc[ni][mi][v] is output column n = wn*WN + ni*32 + 8*(v/4) + 4*(lane/32) + v%4 of output row
-        // m = wm*WM + mi*32 + lane%32: a lane owns 4 consecutive columns of 16 rows per 32x32 block.
-        // Bias, activation and the rounding to Element happen in registers; the wavefront then
-        // transposes 32-row x 64-column panels through a private LDS region (rows of 128 bytes,
-        // 16-byte chunk c of row r at position c ^ ((r >> 1) & 7)) so that the global stores are
-        // 16 bytes per lane and cover whole 128-byte lines of the output rows. The bias comes from
-        // the tile's LDS slot: the epilogue issues no global load, so nothing in it ever waits for
-        // the stores it has in flight.
-        const uint32_t tid = local_tid();
-        const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
-        const int wm = wave / WAVES_N, wn = wave % WAVES_N;
-        const int fr_row = lane & 31, fr_half = lane >> 5;
-        char* stg = stage_mem + wave * (kPanelRows * 128);
-        const char* bias_lane = bias_mem + (wn * WN + 4 * fr_half) * 2;
-#pragma unroll
-        for (int mi = 0; mi < TM; ++mi) {
-#pragma unroll
-            for (int pn = 0; pn < WN / 64; ++pn) {
-#pragma unroll
-                for (int nl = 0; nl < 2; ++nl) {
-                    const int ni = pn * 2 + nl;
-#pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        const vec4 b4 = *reinterpret_cast<const vec4*>(bias_lane + (ni * 32 + 8 * q) * 2);
-                        vec4 o;
-#pragma unroll
-                        for (int j = 0; j < 4; ++j)
-                            o[j] = static_cast<E>(activate<ACT>(acc[ni][mi][4 * q + j] + float(b4[j])));
-                        *reinterpret_cast<vec4*>(stg + fr_row * 128 + (((nl * 4 + q) ^ ((fr_row >> 1) & 7)) << 4) + fr_half * 8) = o;
-                    }
-                }
-                // the same wavefront wrote and reads the region: LDS operations of one wavefront
-                // complete in order
-#pragma unroll
-                for (int it = 0; it < kPanelRows * 8 / kWave; ++it) {
-                    const int id = it * kWave + lane;
-                    const int r = id >> 3, c = id & 7;
-                    const u32x4 v = load16(stg + r * 128 + ((c ^ ((r >> 1) & 7)) << 4));
-                    const uint32_t m = wm * WM + mi * 32 + r, n = wn * WN + pn * 64 + c * 8;
-                    if (m < t.m_valid && n < t.n_valid) store16(t.c_base + size_t(m) * t.ldc + n, v);
-                }
-            }
-        }
-    }
-
     // Epilogue. Every wavefront must have left mainloop().
     static __device__ __forceinline__ void finish(const Tile& t, Acc& acc, char* smem) {
-        char* stage_mem = smem + last_stage(t) * kStage;
-        const char* bias_mem = smem + kBiasOffset + t.bias_slot * kBiasBytes;
-        if (t.act == 0) finish_act<0>(t, acc, stage_mem, bias_mem);
-        else if (t.act == 1) finish_act<1>(t, acc, stage_mem, bias_mem);
-        else finish_act<2>(t, acc, stage_mem, bias_mem);
+        const TileOut out{t.c_base, t.ldc, t.m_valid, t.n_valid, t.act};
+        epilogue16<E, WM, WN, WAVES_N>(out, acc, smem + last_stage(t) * kStage, smem + kBiasOffset + t.bias_slot * kBiasBytes);
     }
 };
 

@@ -30,7 +30,8 @@ constexpr int kXcds = 8;
 // at the headline shape, so its weights stream from HBM exactly once), 2 x 4 wavefronts of 128 x 64
 // (two per SIMD), K slices of 64 (whole 128-byte lines of every row) through two 64 KB stages.
 // (Measured against it on MI355X, none faster: K slices of 32 through four stages, all loads of a
-// slice issued at its first K step, 2 x 2 wavefronts of 128 x 128 with the accumulators in AGPRs.)
+// slice issued at its first K step, 2 x 2 wavefronts of 128 x 128 with the accumulators in AGPRs,
+// weight slices of 64 through three slots with activation half slices of 32 through three.)
 // Variant 1, for layers whose experts hold at most 128 rows (many small experts): a 128 x 256 tile
 // wastes no matrix work and no activation loads on rows that do not exist, and its smaller stages
 // leave room for a third one (measured on the 256-expert top-8 shape: 3.7 ms against 4.6 ms).

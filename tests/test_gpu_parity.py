@@ -134,6 +134,9 @@ CASES = [
     (256, 128, 64, 256, 8, 1.0, 1, 0, 2, 0.0),     # E = 256, top-8
     (256, 128, 192, 8, 2, 1.0, 1, 1, 0, 0.1),      # fp32 + gelu
     (256, 64, 64, 24, 3, 1.0, 1, 0, 0, 0.0),       # fp32, E = 24
+    (1024, 192, 320, 4, 2, 1.0, 1, 0, 2, 0.1),     # 512 rows per expert: 256-row tiles, odd slice counts
+    (512, 64, 64, 2, 1, 1.0, 1, 1, 2, 0.1),        # 256-row tiles over a single K slice
+    (768, 128, 192, 2, 2, 1.0, 1, 0, 3, 0.0),      # fp16, 256-row tiles, a partial row block
     (256, 128, 256, 8, 2, 1.0, 1, 0, 3, 0.0),      # fp16
     (256, 192, 320, 12, 3, 1.0, 1, 1, 3, 0.1),     # fp16, gelu + biases, ragged sizes
     (512, 256, 256, 64, 2, 1.0, 1, 0, 3, 0.0),     # fp16, E = 64, several K slices
