@@ -36,3 +36,13 @@ def oracle():
     from oracle import moe_ref
     moe_ref.lib()
     return moe_ref
+
+
+@pytest.fixture(scope="session", autouse=True)
+def built_library():
+    """The tests load the library that is built in-tree; only when there is none do they build it
+    (hipcc cross-compiles gfx950 without a GPU)."""
+    from aristos_amd import _capi, build
+    if not os.path.exists(_capi.LIB_PATH):
+        build.build_library()
+    return _capi.LIB_PATH
