@@ -372,6 +372,66 @@ extern "C" int kleos_scheduler_stats(double stats[6]) {
     return KLEOS_OK;
 }
 
+extern "C" int kleos_measure_throughput(uint32_t trials, float* median_ms, float* throughput) {
+    if (int rc = require_ctx("kleos_measure_throughput")) return rc;
+    if (!median_ms || !throughput || trials == 0 || trials > 1024)
+        return fail(KLEOS_EINVAL, "kleos_measure_throughput: need result pointers and 1 <= trials <= 1024");
+    Context& c = *g_ctx;
+    KLEOS_HIP(hipSetDevice(c.device));
+    // One expert at full padded capacity, as the reference's probe (throughput.cuh:104-170):
+    // M = pEC rows, up-projection to I columns over K = H, activation, down-projection back to H.
+    const kleos_config_t& cfg = c.cfg;
+    const size_t eb = cfg.elem_bytes, M = cfg.pEC, H = cfg.H, I = cfg.I;
+    size_t off = 0;
+    auto take = [&](size_t bytes) { size_t o = off; off = align_up(off + bytes, 256); return o; };
+    const size_t o_x = take(M * H * eb), o_wu = take(I * H * eb), o_wd = take(H * I * eb), o_bu = take(I * eb),
+                 o_bd = take(H * eb), o_h1 = take(M * I * eb), o_y = take(M * H * eb), o_cnt = take(4),
+                 o_tok = take(M * 4);
+    char* buf = nullptr;
+    KLEOS_HIP(hipMalloc(reinterpret_cast<void**>(&buf), off));
+    int rc = KLEOS_OK;
+    std::vector<hipEvent_t> ev(size_t(trials) * 2, nullptr);
+    auto body = [&]() -> int {
+        // finite, small operands (every byte 0x3c: 0.0115 in bf16 and fp32, 1.06 in fp16); the
+        // timing does not depend on the values
+        KLEOS_HIP(hipMemsetAsync(buf, 0x3c, o_cnt, c.stream));
+        std::vector<int32_t> tok(M);
+        for (size_t i = 0; i < M; ++i) tok[i] = int32_t(i);
+        const uint32_t count = uint32_t(M);
+        KLEOS_HIP(hipMemcpyAsync(buf + o_cnt, &count, 4, hipMemcpyHostToDevice, c.stream));
+        KLEOS_HIP(hipMemcpyAsync(buf + o_tok, tok.data(), M * 4, hipMemcpyHostToDevice, c.stream));
+        KLEOS_HIP(hipStreamSynchronize(c.stream));
+        LayerParams q{};
+        q.S = uint32_t(M); q.H = cfg.H; q.I = cfg.I; q.E = 1; q.k = 1; q.PX = 64; q.EC = uint32_t(M);
+        q.cap_rows = uint32_t(M); q.act = cfg.hidden_act;
+        q.x = buf + o_x; q.w_up = buf + o_wu; q.w_down = buf + o_wd; q.b_up = buf + o_bu; q.b_down = buf + o_bd;
+        q.h1 = buf + o_h1; q.y = buf + o_y;
+        q.expert_count = reinterpret_cast<uint32_t*>(buf + o_cnt);
+        q.slot_token = reinterpret_cast<int32_t*>(buf + o_tok);
+        const int dt = int(cfg.torch_dtype);
+        for (auto& e : ev) KLEOS_HIP(hipEventCreate(&e));
+        for (uint32_t t = 0; t < trials + 2; ++t) {          // two warm-up rounds
+            const bool timed = t >= 2;
+            if (timed) KLEOS_HIP(hipEventRecord(ev[size_t(t - 2) * 2], c.stream));
+            KLEOS_HIP(launch_expert_gemm(q, dt, 0, c.num_cus, c.stream));
+            KLEOS_HIP(launch_expert_gemm(q, dt, 1, c.num_cus, c.stream));
+            if (timed) KLEOS_HIP(hipEventRecord(ev[size_t(t - 2) * 2 + 1], c.stream));
+        }
+        KLEOS_HIP(hipStreamSynchronize(c.stream));
+        std::vector<float> ms(trials);
+        for (uint32_t t = 0; t < trials; ++t) KLEOS_HIP(hipEventElapsedTime(&ms[t], ev[size_t(t) * 2], ev[size_t(t) * 2 + 1]));
+        std::sort(ms.begin(), ms.end());
+        *median_ms = ms[trials / 2];                          // throughput.cuh:166 (findMedian)
+        *throughput = *median_ms > 0.f ? 1.0f / *median_ms : 0.f;
+        return KLEOS_OK;
+    };
+    rc = body();
+    (void)hipStreamSynchronize(c.stream);
+    for (auto& e : ev) if (e) (void)hipEventDestroy(e);
+    (void)hipFree(buf);
+    return rc;
+}
+
 extern "C" int kleos_gate_loss(float* loss, float* mean_prob, float* mean_count) {
     if (int rc = require_ctx("kleos_gate_loss")) return rc;
     Context& c = *g_ctx;

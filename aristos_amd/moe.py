@@ -56,6 +56,15 @@ def scheduler_stats() -> dict:
     return dict(zip(keys, (float(v) for v in arr)))
 
 
+def measure_throughput(trials: int = 16) -> dict:
+    """One expert at full padded capacity through both projections (the reference's mT probe,
+    throughput.cuh:104-170): median latency in ms and its reciprocal."""
+    ms = C.c_float(0.0)
+    thr = C.c_float(0.0)
+    _capi.check(_capi.lib().kleos_measure_throughput(int(trials), C.byref(ms), C.byref(thr)))
+    return {"median_ms": float(ms.value), "throughput": float(thr.value)}
+
+
 def gate_loss(n_experts: int) -> dict:
     """Training mode: loss, mean probability [E] and mean routed count [E] of the last forward."""
     loss = C.c_float(0.0)

@@ -171,6 +171,13 @@ int kleos_phase_times(float ms[5]);
  * unfinished dependency, publishing finished tiles; [3] expert tiles executed; [4] tiles handed out
  * before their inputs were complete; [5] tiles taken from another XCD's queue. */
 int kleos_scheduler_stats(double stats[6]);
+/* Replaces kleos::mT (csrc/include/kleos/throughput.cuh:104-170), the probe the reference runs at
+ * start-up to rate a device: one expert at full padded capacity (pEC rows) through the up-projection,
+ * activation and down-projection of the configured sizes, `trials` times on the library stream after
+ * two warm-up rounds. *median_ms receives the median latency of a round, *throughput its reciprocal
+ * (experts per millisecond), the figure the reference stores in WorkerAttribute::throughput. Allocates
+ * and frees its own operands; the context's state is untouched. */
+int kleos_measure_throughput(uint32_t trials, float* median_ms, float* throughput);
 /* Training mode (is_training: 1): the load-balancing loss of the gate of the most recent forward,
  * which the reference leaves in its bookkeeping arena (gML, gMeC, gL; csrc/include/kleos/types.cuh:
  * 940-958, computed at moe/gate.cuh:608-635, 700-705, 763-773): mean_prob[e] = mean over the tokens

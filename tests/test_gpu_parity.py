@@ -417,3 +417,26 @@ def test_cpp_driver_prints_the_reference_line(tmp_path):
     assert r.returncode == 0, r.stderr
     m = re.search(r"epRank: 0 took ([0-9.]+)\s*ms", r.stdout)
     assert m and float(m.group(1)) > 0, r.stdout
+
+
+def test_throughput_probe_leaves_the_context_alone():
+    """kleos_measure_throughput (the reference's mT, throughput.cuh:104-170) times one expert at
+    padded capacity on its own buffers; a forward before and after it gives the same bits."""
+    keys = _keys(1024, 256, 512, 8, 2)
+    c = moe_ref.cfg_from_keys(keys)
+    x, wg, w_up, w_down, *_ = random_layer(c, seed=51, w_std=0.05)
+    iP = _to_device(c, pack_inputs(c, x, wg, w_up, w_down))
+    d = ka.initialize(keys)
+    try:
+        oP = synth.alloc_outputs(d)
+        ka.moe.forward_host(iP, oP)
+        ka.moe.stream_synchronize()
+        before = _out_to_np(c, oP).copy()
+        r = ka.moe.measure_throughput(8)
+        assert r["median_ms"] > 0 and abs(r["throughput"] * r["median_ms"] - 1.0) < 1e-5
+        oP.fill_(float("nan"))
+        ka.moe.forward_host(iP, oP)
+        ka.moe.stream_synchronize()
+        np.testing.assert_array_equal(_out_to_np(c, oP), before)
+    finally:
+        ka.finalize()
