@@ -18,11 +18,12 @@ import ctypes as _C
 import os as _os
 
 from . import _capi, moe
-from ._capi import KleosError, MODE_FUSED, MODE_PHASED, DTYPE_FP32, DTYPE_BF16, ACT_RELU, ACT_GELU
+from ._capi import KleosError, MODE_FUSED, MODE_PHASED, SCHEDULE_AUTO, SCHEDULE_DYNAMIC, SCHEDULE_STATIC, DTYPE_FP32, DTYPE_BF16, ACT_RELU, ACT_GELU
 from .config import KleosConfig, DerivedConfig
 
 __all__ = ["initialize", "finalize", "is_initialized", "get_rank", "set_device", "active_config", "moe",
-           "KleosConfig", "DerivedConfig", "KleosError", "MODE_FUSED", "MODE_PHASED"]
+           "KleosConfig", "DerivedConfig", "KleosError", "MODE_FUSED", "MODE_PHASED",
+           "SCHEDULE_AUTO", "SCHEDULE_DYNAMIC", "SCHEDULE_STATIC"]
 
 
 def initialize(config) -> DerivedConfig:

@@ -11,6 +11,7 @@ KLEOS_OK, KLEOS_EINVAL, KLEOS_ESTATE, KLEOS_EUNSUPPORTED, KLEOS_EHIP, KLEOS_EIO,
 DTYPE_FP32, DTYPE_TF32, DTYPE_BF16, DTYPE_FP16 = range(4)
 ACT_RELU, ACT_GELU = 0, 1
 MODE_FUSED, MODE_PHASED = 0, 1
+SCHEDULE_AUTO, SCHEDULE_DYNAMIC, SCHEDULE_STATIC = 0, 1, 2
 
 
 class KleosConfigStruct(C.Structure):
@@ -57,6 +58,9 @@ SYMBOLS = {
     "kleos_stream": (C.c_void_p, []),
     "kleos_set_mode": (C.c_int, [C.c_int]),
     "kleos_get_mode": (C.c_int, []),
+    "kleos_set_schedule": (C.c_int, [C.c_int]),
+    "kleos_get_schedule": (C.c_int, []),
+    "kleos_schedule_taken": (C.c_int, [C.POINTER(C.c_int)]),
     "kleos_moe_debug_views": (C.c_int, [C.POINTER(DebugViewsStruct)]),
     "kleos_debug_copy_to_host": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t]),
     "kleos_scheduler_stats": (C.c_int, [C.POINTER(C.c_double)]),

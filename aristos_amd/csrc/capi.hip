@@ -28,6 +28,7 @@ struct Context {
     uint32_t launch_seq = 0;        // forwards issued, any mode (parity selects the live coarse counts)
     uint32_t fused_seq = 0;         // fused forwards issued (grid-barrier arrival base)
     int mode = KLEOS_MODE_FUSED;
+    int schedule = KLEOS_SCHEDULE_AUTO;
     float phase_ms[5] = {0, 0, 0, 0, 0};
     double sched_stats[6] = {0, 0, 0, 0, 0, 0};
 };
@@ -125,7 +126,7 @@ int enqueue_forward(Context& c, const void* iP, void* oP, hipEvent_t* ev) {
     p.epoch = c.launch_seq++;
     const int dt = int(c.cfg.torch_dtype);
     if (c.mode == KLEOS_MODE_FUSED) {
-        KLEOS_HIP(launch_fused(p, c.plan, c.fused_seq++, c.stream));
+        KLEOS_HIP(launch_fused(p, c.plan, c.fused_seq++, c.schedule, c.stream));
         return KLEOS_OK;
     }
     if (ev) KLEOS_HIP(hipEventRecord(ev[0], c.stream));
@@ -263,6 +264,29 @@ extern "C" int kleos_set_mode(int mode) {
 }
 
 extern "C" int kleos_get_mode(void) { return g_ctx ? g_ctx->mode : -1; }
+
+extern "C" int kleos_set_schedule(int schedule) {
+    if (int rc = require_ctx("kleos_set_schedule")) return rc;
+    if (schedule != KLEOS_SCHEDULE_AUTO && schedule != KLEOS_SCHEDULE_DYNAMIC && schedule != KLEOS_SCHEDULE_STATIC)
+        return fail(KLEOS_EINVAL, "kleos_set_schedule: unknown schedule %d", schedule);
+    g_ctx->schedule = schedule;
+    return KLEOS_OK;
+}
+
+extern "C" int kleos_get_schedule(void) { return g_ctx ? g_ctx->schedule : -1; }
+
+extern "C" int kleos_schedule_taken(int* schedule) {
+    if (int rc = require_ctx("kleos_schedule_taken")) return rc;
+    if (!schedule) return fail(KLEOS_EINVAL, "kleos_schedule_taken: null argument");
+    Context& c = *g_ctx;
+    if (c.fused_seq == 0) return fail(KLEOS_ESTATE, "kleos_schedule_taken: no persistent launch yet");
+    KLEOS_HIP(hipSetDevice(c.device));
+    KLEOS_HIP(hipStreamSynchronize(c.stream));
+    unsigned long long flag = 0;   // workgroup 0, word 14 of its stamp row
+    KLEOS_HIP(hipMemcpy(&flag, c.base.stamps + 14, sizeof(flag), hipMemcpyDeviceToHost));
+    *schedule = flag ? KLEOS_SCHEDULE_STATIC : KLEOS_SCHEDULE_DYNAMIC;
+    return KLEOS_OK;
+}
 
 extern "C" int kleos_moe_forward(const void* iP, void* oP) {
     if (int rc = require_ctx("kleos_moe_forward")) return rc;

@@ -76,11 +76,20 @@ __device__ __forceinline__ uint32_t kept_rows(const LayerParams& p, uint32_t e) 
 //   kSchedBar + 32 b              grid barrier b: groups that have arrived, monotonic across launches
 //   kSchedGroup + 32 (8 b + g)    grid barrier b: arrivals of workgroup group g, monotonic
 //   kSchedTicket + 32 q           ticket counter of XCD queue q
+//   kSchedMembers + 32 (8 h + x)  workgroups of this launch that run on XCD x; h = launch parity
 //   kSchedReady + e*mt_max + m    readiness: up-projection tiles stored per (expert, row block)
 //   kSchedError                   set to non-zero by a workgroup whose bounded wait expired
+//   kSchedStaticRuns              launches so far that took the static schedule (they hold one more
+//                                 grid barrier, whose arrival counters advance only with them)
 constexpr uint32_t kSchedLine = 32;
-constexpr uint32_t kSchedBar = 0, kSchedError = 4, kSchedTicket = 4 * kSchedLine, kSchedGroup = 12 * kSchedLine,
-                   kSchedReady = 36 * kSchedLine;
+constexpr uint32_t kSchedBar = 0, kSchedError = 4, kSchedStaticRuns = 5, kSchedTicket = 4 * kSchedLine,
+                   kSchedGroup = 12 * kSchedLine, kSchedMembers = 44 * kSchedLine, kSchedReady = 60 * kSchedLine;
+constexpr uint32_t kGridBarriers = 4;
+// schedule of the expert phase of the persistent kernel (the values of kleos_amd.h's KLEOS_SCHEDULE_*)
+constexpr uint32_t kScheduleAuto = 0, kScheduleStatic = 2;   // anything else: dynamic
+static_assert(kSchedBar + kGridBarriers * kSchedLine <= kSchedTicket, "barrier words");
+static_assert(kSchedGroup + kGridBarriers * kXcds * kSchedLine <= kSchedMembers, "barrier group words");
+static_assert(kSchedMembers + 2 * kXcds * kSchedLine <= kSchedReady, "member words");
 // Every wait in the persistent kernel is bounded so that the grid always drains: after this many
 // ticks of the 100 MHz wall clock a waiter records an error and proceeds.
 constexpr unsigned long long kWaitTicks = 300000000ull;   // 3 s
@@ -138,6 +147,26 @@ __device__ __forceinline__ void grid_barrier(uint32_t* sched, uint32_t which, ui
     asm volatile("buffer_inv sc0" ::: "memory");
 }
 
+// Barrier among the `members` workgroups that run on XCD `xcd`, the `runs`-th time it is held on this
+// arena (counted from 0). The static schedule holds it between the two projections: a down tile
+// reads h1 rows that only workgroups of its own XCD stored.
+__device__ __forceinline__ void xcd_barrier(uint32_t* sched, uint32_t xcd, uint32_t runs, uint32_t members) {
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        uint32_t* arrived = sched + kSchedGroup + ((kGridBarriers - 1) * kXcds + xcd) * kSchedLine;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+        atomic_add_agent(arrived, 1u);
+        const uint32_t target = (runs + 1u) * members;
+        bounded_wait(sched, [&] { return int32_t(atomic_load_relaxed(arrived) - target) >= 0; });
+    }
+    __syncthreads();
+    asm volatile("buffer_inv sc0" ::: "memory");   // drop this CU's L1; the rows are current in the XCD's L2
+}
+
+__device__ __forceinline__ bool balanced_or_forced(uint32_t policy, bool balanced) {
+    return policy == kScheduleStatic || (policy == kScheduleAuto && balanced);
+}
+
 // One unit of expert work: an output tile of the up-projection (kind 0: h1 = act(x_gathered *
 // Wup^T + bup)) or of the down-projection (kind 1: y = h1 * Wdown^T + bdown, identity activation,
 // types.cuh:461). The reference's 128-byte Task descriptor (types.cuh:565-654) shrinks to this.
@@ -148,6 +177,7 @@ struct Task {
     uint32_t dep;       // down tile: the readiness counter of its row block as seen when handed out
     uint32_t ready;     // down tile whose up-projection row block was already complete when handed out
     uint32_t valid;
+    uint32_t sync;      // not a tile (valid == 0): hold the grid barrier of the static schedule, then ask again
 };
 constexpr int kTaskWords = 12;
 
@@ -157,13 +187,13 @@ __device__ __forceinline__ Task broadcast_task(uint32_t* s_task, const Task& min
     if (threadIdx.x == 0) {
         s_task[0] = mine.e; s_task[1] = mine.kind; s_task[2] = mine.mtile; s_task[3] = mine.ntile;
         s_task[4] = mine.foreign; s_task[5] = mine.ready; s_task[6] = mine.valid; s_task[7] = mine.rows;
-        s_task[8] = mine.dep;
+        s_task[8] = mine.dep; s_task[9] = mine.sync;
     }
     __syncthreads();
     Task t;
     t.e = s_task[0]; t.kind = s_task[1]; t.mtile = s_task[2]; t.ntile = s_task[3];
     t.foreign = s_task[4]; t.ready = s_task[5]; t.valid = s_task[6]; t.rows = s_task[7];
-    t.dep = s_task[8];
+    t.dep = s_task[8]; t.sync = s_task[9];
     return t;
 }
 
@@ -215,9 +245,11 @@ struct Readiness {
 // `stats` (thread 0 only, may be null) accumulates 100 MHz ticks spent [0] fetching tasks,
 // [1] waiting for a dependency, [2] publishing, and counts [3] tiles, [4] tiles handed out before
 // their inputs were complete, [5] tiles taken from a foreign queue.
-template <typename T, int V, typename Next>
+// `mid_sync()` is called by every thread when `next` hands out a sync marker (static schedule
+// only: once per workgroup, between its last up tile and its first down tile).
+template <typename T, int V, typename Next, typename Sync>
 __device__ __forceinline__ void expert_loop(const LayerParams& p, char* smem, uint32_t* s_task, const Readiness rd,
-                                            unsigned long long* stats, Next&& next_raw) {
+                                            unsigned long long* stats, Next&& next_raw, Sync&& mid_sync) {
     const uint32_t tid = threadIdx.x;
     unsigned long long st_next = 0, st_wait = 0, st_pub = 0, n_tiles = 0, n_late = 0, n_foreign = 0;
     auto next = [&]() {
@@ -279,6 +311,7 @@ __device__ __forceinline__ void expert_loop(const LayerParams& p, char* smem, ui
         typename G::Tile cur_t, nxt_t;
         typename G::Acc acc;
         Task cur = next();
+        if (cur.sync) { mid_sync(); cur = next(); }
         if (!cur.valid) { flush_stats(); return; }
         if (cur.kind == 1 && !cur.ready) wait_ready(cur);
         acquire(cur);
@@ -301,9 +334,10 @@ __device__ __forceinline__ void expert_loop(const LayerParams& p, char* smem, ui
                 __syncthreads();
                 publish(cur);
             }
+            if (nxt.sync) { mid_sync(); nxt = next(); }
             if (!nxt.valid) break;
             if (!early) {
-                wait_ready(nxt);
+                if (nxt.kind == 1 && !nxt.ready) wait_ready(nxt);
                 acquire(nxt);
                 G::begin(nxt_t, args_of(nxt), G::next_stage0(cur_t), bias_slot ^= 1, smem);
             }
@@ -314,6 +348,7 @@ __device__ __forceinline__ void expert_loop(const LayerParams& p, char* smem, ui
     } else {
         for (;;) {
             Task t = next();
+            if (t.sync) { mid_sync(); continue; }
             if (!t.valid) break;
             if (t.kind == 1 && !t.ready) wait_ready(t);
             acquire(t);
@@ -384,7 +419,7 @@ __global__ __launch_bounds__((TileShape<T, V>::kThreads), (TileShape<T, V>::kPer
         }
         return broadcast_task(s_task, t);
     };
-    expert_loop<T, V>(p, gemm_smem + kPhasedGemmHeader, s_task, Readiness{nullptr, 0, 0}, nullptr, next);
+    expert_loop<T, V>(p, gemm_smem + kPhasedGemmHeader, s_task, Readiness{nullptr, 0, 0}, nullptr, next, [] {});
 }
 
 template <typename T>
@@ -397,7 +432,7 @@ __global__ __launch_bounds__(kPhaseThreads) void combine_kernel(const LayerParam
 // ------------------------------------------------------------------------------------ fused
 template <typename T, int NG, int V>
 __global__ __launch_bounds__((TileShape<T, V>::kThreads), (TileShape<T, V>::kPerCu)) void fused_kernel(const LayerParams p, uint32_t seq,
-                                                                      uint32_t mt_max, uint32_t lag) {
+                                                                      uint32_t mt_max, uint32_t dynamic_lag, uint32_t policy) {
     static_assert(sizeof(Segment) == 8, "segment table sizing");
     extern __shared__ __attribute__((aligned(16))) char smem[];
     constexpr int BM = TileShape<T, V>::BM, BN = TileShape<T, V>::BN;
@@ -409,10 +444,25 @@ __global__ __launch_bounds__((TileShape<T, V>::kThreads), (TileShape<T, V>::kPer
     unsigned long long* stamp = p.stamps + size_t(blockIdx.x) * kStampWords;
     if (tid == 0) stamp[0] = wall_clock64();
 
-    // ---- phase 0: gate. Workgroup 0 also resets this launch's tickets and readiness counters;
-    // nothing reads them before the second barrier.
+    // The XCD this workgroup really runs on (hardware register XCC_ID): expert e's tiles are queued
+    // on XCD e % 8, so that its weights, its gathered rows and the h1 rows handed from its
+    // up-projection to its down-projection all live in one L2. Every workgroup also takes a rank
+    // among the workgroups of its XCD, which the static schedule strides by.
+    const uint32_t xcd = __builtin_amdgcn_s_getreg((3 << 11) | 20) & (kXcds - 1);
+    uint32_t* const members_now = sched + kSchedMembers + (seq & 1u) * kXcds * kSchedLine;
+    uint32_t my_rank = 0, static_runs = 0;
+    if (tid == 0) {
+        my_rank = atomic_add_agent(members_now + xcd * kSchedLine, 1u);
+        static_runs = atomic_load_relaxed(sched + kSchedStaticRuns);
+    }
+
+    // ---- phase 0: gate. Workgroup 0 also resets this launch's tickets and readiness counters
+    // (nothing reads them before the second barrier) and the next launch's member counts.
     if (blockIdx.x == 0) {
-        if (tid < uint32_t(kXcds)) sched[kSchedTicket + tid * kSchedLine] = 0u;
+        if (tid < uint32_t(kXcds)) {
+            sched[kSchedTicket + tid * kSchedLine] = 0u;
+            sched[kSchedMembers + (((seq + 1u) & 1u) * kXcds + tid) * kSchedLine] = 0u;
+        }
         for (uint32_t i = tid; i < p.E * mt_max; i += kThreads) sched[kSchedReady + i] = 0u;
     }
     for (uint32_t unit = blockIdx.x; unit < ceil_div_u32(p.n_gate_tiles, gate_unit_blocks<NG>()); unit += nwg)
@@ -441,54 +491,125 @@ __global__ __launch_bounds__((TileShape<T, V>::kThreads), (TileShape<T, V>::kPer
     uint32_t* s_qseg = reinterpret_cast<uint32_t*>(smem + kLdsMt);              // [9] first segment of each queue
     uint32_t* s_qtot = s_qseg + 16;                                             // [8] tickets in each queue
     uint32_t* s_task = s_qtot + 8;                                              // [kTaskWords] task broadcast slot
+    uint32_t* s_qup = s_task + kTaskWords;                                      // [8] up-projection tickets in each queue
+    // static schedule: [1] rank of the workgroup among those of its XCD,
+    // [2] static launches before this one, [3] next ticket of the workgroup, [4] the barrier between
+    // the projections is behind, [5] every XCD holds the same number of workgroups. Thread 0's own words live here rather than in registers that would
+    // stay occupied through the GEMM main loop.
+    uint32_t* s_static = s_qup + 8;
+    static_assert((16 + 8 + kTaskWords + 8 + 6) * 4 <= kLdsQueue, "queue header");
     Segment* s_seg = reinterpret_cast<Segment*>(smem + kLdsMt + kLdsQueue);     // at most 2*E segments
     char* s_gemm = smem + kFusedLdsHeader;
     const uint32_t tn_up = ceil_div_u32(p.I, BN), tn_down = ceil_div_u32(p.H, BN);
 
+    // how many workgroups every XCD holds: asked for first, so that the answers travel together
+    // with the routed counts below
+    uint32_t seen[kXcds] = {};
+    if (tid == 0)
+        for (uint32_t j = 0; j < kXcds; ++j) seen[j] = atomic_load_relaxed(members_now + j * kSchedLine);
     for (uint32_t e = tid; e < p.E; e += kThreads) {
         const uint32_t rows = kept_rows<true>(p, e);
         s_rows[e] = rows;
         s_mt[e] = uint16_t(ceil_div_u32(rows, BM));
     }
     __syncthreads();
+    const uint32_t members = nwg / kXcds;
+    // Static or dynamic schedule: every workgroup decides alike, from the same counters.
+    // Static: each XCD's workgroups stride through their queue's up tiles, meet at a barrier, then
+    // stride through its down tiles: no tickets, no readiness counters, no per-tile publication.
+    // It needs every XCD to hold the same number of workgroups, and it pays only when the queues
+    // hold about the same work (nobody to steal from).
+    // Thread q sets up queue q; its segments start at a fixed place, two per expert of the queue.
+    const uint32_t my_nq = tid < p.E && tid < uint32_t(kXcds) ? (p.E - tid + kXcds - 1) / kXcds : 0u;   // experts q, q+8, ...
+    if (tid < uint32_t(kXcds)) {
+        uint32_t blocks = 0;
+        for (uint32_t i = 0; i < my_nq; ++i) blocks += s_mt[tid + kXcds * i];
+        s_qtot[tid] = blocks;
+    }
     if (tid == 0) {
-        uint32_t nseg = 0;
-        for (uint32_t q = 0; q < kXcds; ++q) {
-            s_qseg[q] = nseg;
-            const uint32_t nq = q < p.E ? (p.E - q + kXcds - 1) / kXcds : 0u;   // experts q, q+8, ...
-            uint32_t ticket = 0;
-            // up-projection of expert i, then down-projection of expert i - lag: a down tile is
-            // handed out only after `lag` further experts' worth of tickets, by which time the
-            // up tiles it depends on have normally been stored.
-            for (uint32_t i = 0; i < nq + lag; ++i) {
-                if (i < nq) {
-                    const uint32_t e = q + kXcds * i;
-                    s_seg[nseg++] = Segment{uint16_t(e), 0, 0, ticket};
-                    ticket += uint32_t(s_mt[e]) * tn_up;
-                }
-                if (i >= lag) {
-                    const uint32_t e = q + kXcds * (i - lag);
-                    s_seg[nseg++] = Segment{uint16_t(e), 1, 0, ticket};
-                    ticket += uint32_t(s_mt[e]) * tn_down;
-                }
-            }
-            s_qtot[q] = ticket;
-        }
-        s_qseg[kXcds] = nseg;
+        bool even = nwg % kXcds == 0;
+        for (uint32_t j = 0; j < kXcds; ++j) even = even && seen[j] == members;
+        s_static[1] = my_rank;
+        s_static[2] = static_runs;
+        s_static[3] = my_rank;
+        s_static[4] = 0u;
+        s_static[5] = even;
     }
     __syncthreads();
+    bool use_static;
+    {
+        uint32_t lo = ~0u, hi = 0;
+        for (uint32_t q = 0; q < kXcds; ++q) {
+            const uint32_t blocks = s_qtot[q];
+            lo = blocks < lo ? blocks : lo;
+            hi = blocks > hi ? blocks : hi;
+        }
+        const bool balanced = hi - lo <= hi / 16;
+        // the same in every lane: keep it in a scalar register
+        use_static = __builtin_amdgcn_readfirstlane(int(s_static[5] != 0 && balanced_or_forced(policy, balanced))) != 0;
+    }
+    __syncthreads();   // the row-block sums above shared s_qtot with the ticket totals below
+    if (tid < uint32_t(kXcds)) {
+        const uint32_t q = tid, nq = my_nq;
+        const uint32_t first = 2 * (q * (p.E / kXcds) + (q < p.E % kXcds ? q : p.E % kXcds));
+        uint32_t nseg = first;
+        s_qseg[q] = first;
+        if (q == kXcds - 1) s_qseg[kXcds] = 2 * p.E;
+        const uint32_t lag = use_static ? nq : dynamic_lag;   // static: all ups, then all downs
+        uint32_t ticket = 0, ups = 0;
+        // up-projection of expert i, then down-projection of expert i - lag: a down tile is
+        // handed out only after `lag` further experts' worth of tickets, by which time the
+        // up tiles it depends on have normally been stored.
+        for (uint32_t i = 0; i < nq + lag; ++i) {
+            if (i < nq) {
+                const uint32_t e = q + kXcds * i;
+                s_seg[nseg++] = Segment{uint16_t(e), 0, 0, ticket};
+                ticket += uint32_t(s_mt[e]) * tn_up;
+                ups += uint32_t(s_mt[e]) * tn_up;
+            }
+            if (i >= lag && i - lag < nq) {
+                const uint32_t e = q + kXcds * (i - lag);
+                s_seg[nseg++] = Segment{uint16_t(e), 1, 0, ticket};
+                ticket += uint32_t(s_mt[e]) * tn_down;
+            }
+        }
+        s_qtot[q] = ticket;
+        s_qup[q] = ups;
+    }
+    __syncthreads();
+    if (tid == 0) stamp[14] = use_static;
 
-    // The XCD this workgroup really runs on (hardware register XCC_ID): expert e's tiles are queued
-    // on XCD e % 8, so that its weights, its gathered rows and the h1 rows handed from its
-    // up-projection to its down-projection all live in one L2.
-    const uint32_t xcd = __builtin_amdgcn_s_getreg((3 << 11) | 20) & (kXcds - 1);
     uint32_t q_off = 0;   // queues already found empty, starting from this workgroup's own XCD
     uint32_t q_dead = 0;  // bit q: queue q was seen exhausted
     bool q_scanned = false;
-    const Readiness rd{sched, mt_max, tn_up};
+    const Readiness rd{use_static ? nullptr : sched, mt_max, tn_up};
+    auto decode = [&](Task& t, uint32_t q, uint32_t ticket) {
+        uint32_t sg = s_qseg[q];
+        const uint32_t sg_end = s_qseg[q + 1];
+        while (sg + 1 < sg_end && s_seg[sg + 1].start <= ticket) ++sg;
+        t.e = s_seg[sg].expert;
+        t.kind = s_seg[sg].kind;
+        const uint32_t local = ticket - s_seg[sg].start;
+        t.mtile = local % s_mt[t.e];
+        t.ntile = local / s_mt[t.e];
+        t.rows = s_rows[t.e];
+        t.valid = 1;
+    };
     auto next = [&]() {
         Task t{};
-        if (tid == 0) {
+        if (tid == 0 && use_static) {
+            const uint32_t ticket = s_static[3];
+            const bool down = s_static[4] != 0;
+            if (!down && ticket >= s_qup[xcd]) {
+                s_static[4] = 1u;
+                s_static[3] = s_qup[xcd] + s_static[1];
+                t.sync = 1;
+            } else if (ticket < (down ? s_qtot[xcd] : s_qup[xcd])) {
+                decode(t, xcd, ticket);
+                t.ready = 1;
+                s_static[3] = ticket + members;
+            }
+        } else if (tid == 0) {
             while (q_off < kXcds) {
                 const uint32_t q = (xcd + q_off) % kXcds;
                 if (q_off != 0 && !q_scanned) {
@@ -503,28 +624,21 @@ __global__ __launch_bounds__((TileShape<T, V>::kThreads), (TileShape<T, V>::kPer
                 if (s_qtot[q] == 0 || ((q_dead >> q) & 1u)) { ++q_off; continue; }
                 const uint32_t ticket = atomic_add_agent(sched + kSchedTicket + q * kSchedLine, 1u);
                 if (ticket >= s_qtot[q]) { ++q_off; continue; }
-                uint32_t sg = s_qseg[q];
-                const uint32_t sg_end = s_qseg[q + 1];
-                while (sg + 1 < sg_end && s_seg[sg + 1].start <= ticket) ++sg;
-                t.e = s_seg[sg].expert;
-                t.kind = s_seg[sg].kind;
-                const uint32_t local = ticket - s_seg[sg].start;
-                t.mtile = local % s_mt[t.e];
-                t.ntile = local / s_mt[t.e];
-                t.rows = s_rows[t.e];
+                decode(t, q, ticket);
                 t.foreign = q_off != 0;
                 t.dep = t.kind == 0 ? 0u : atomic_load_relaxed(rd.counter(t));
                 t.ready = t.kind == 0 || rd.complete(t.dep);
-                t.valid = 1;
                 break;
             }
         }
         return broadcast_task(s_task, t);
     };
-    expert_loop<T, V>(p, s_gemm, s_task, rd, stamp + 8, next);
+    expert_loop<T, V>(p, s_gemm, s_task, rd, stamp + 8, next, [&] { xcd_barrier(sched, xcd, s_static[2], members); });
     if (tid == 0) stamp[5] = wall_clock64();
     grid_barrier(sched, 2, seq, nwg);
     if (tid == 0) stamp[6] = wall_clock64();
+    // every workgroup read the count when it started, before the first barrier
+    if (use_static && blockIdx.x == 0 && tid == 0) atomic_store_relaxed(sched + kSchedStaticRuns, s_static[2] + 1u);
 
     // ---- phase 3: combine, one token per wavefront
     if (p.is_training && blockIdx.x == nwg - 1 && wave == kWaves - 1) gate_loss_finalize(p);
@@ -704,11 +818,11 @@ hipError_t plan_fused(const LayerParams& p, int dtype, int num_cus, FusedPlan* p
     });
 }
 
-hipError_t launch_fused(const LayerParams& p, const FusedPlan& plan, uint32_t fused_seq, hipStream_t s) {
+hipError_t launch_fused(const LayerParams& p, const FusedPlan& plan, uint32_t fused_seq, int schedule, hipStream_t s) {
     uint32_t seq = fused_seq;
-    uint32_t mt_max = plan.mt_max, lag = plan.lag;
+    uint32_t mt_max = plan.mt_max, lag = plan.lag, policy = uint32_t(schedule);
     LayerParams pc = p;
-    void* args[] = {&pc, &seq, &mt_max, &lag};
+    void* args[] = {&pc, &seq, &mt_max, &lag, &policy};
     return hipLaunchKernel(plan.kernel, dim3(plan.nwg), dim3(plan.threads), args, plan.smem, s);
 }
 

@@ -29,7 +29,8 @@ struct FusedPlan {
 };
 hipError_t plan_fused(const LayerParams& p, int dtype, int num_cus, FusedPlan* plan);
 // fused_seq: number of fused launches already issued on this scheduler arena.
-hipError_t launch_fused(const LayerParams& p, const FusedPlan& plan, uint32_t fused_seq, hipStream_t s);
+// schedule: a KLEOS_SCHEDULE_* value.
+hipError_t launch_fused(const LayerParams& p, const FusedPlan& plan, uint32_t fused_seq, int schedule, hipStream_t s);
 
 // Why a configuration cannot run, or nullptr when it can.
 const char* unsupported_reason(uint32_t E, uint32_t k);

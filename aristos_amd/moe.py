@@ -41,6 +41,19 @@ def set_mode(mode: int) -> None:
     _capi.check(_capi.lib().kleos_set_mode(int(mode)))
 
 
+def set_schedule(schedule: int) -> None:
+    """SCHEDULE_AUTO (default), SCHEDULE_DYNAMIC or SCHEDULE_STATIC: how the persistent launch hands
+    out expert tiles."""
+    _capi.check(_capi.lib().kleos_set_schedule(int(schedule)))
+
+
+def schedule_taken() -> int:
+    """SCHEDULE_DYNAMIC or SCHEDULE_STATIC: what the most recent persistent launch did."""
+    out = C.c_int(-1)
+    _capi.check(_capi.lib().kleos_schedule_taken(C.byref(out)))
+    return int(out.value)
+
+
 def phase_times() -> dict:
     """Per-phase milliseconds of the last phased forward_host_bench."""
     arr = (C.c_float * 5)()

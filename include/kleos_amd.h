@@ -138,6 +138,22 @@ enum { KLEOS_MODE_FUSED = 0, KLEOS_MODE_PHASED = 1 };
 int kleos_set_mode(int mode);
 int kleos_get_mode(void);
 
+/* How the persistent launch hands out expert tiles. The reference's scheduler is dynamic only
+ * (csrc/include/kleos/os/scheduler.cuh); here the dynamic schedule (per-XCD ticket queues, readiness
+ * counters, work stealing) has a static sibling: each XCD's workgroups stride through the
+ * up-projection tiles of their queue, the grid meets at a barrier, and they stride through the
+ * down-projection tiles. It spends nothing per tile on tickets and publication, and loses when the
+ * queues hold unequal work. KLEOS_SCHEDULE_AUTO (default) decides inside the kernel, from the
+ * routed counts of the launch: static when the row blocks per queue differ by at most 1/16.
+ * KLEOS_SCHEDULE_STATIC still falls back to the dynamic schedule when the hardware did not place
+ * the same number of workgroups on every XCD. Outputs are identical under every schedule. */
+enum { KLEOS_SCHEDULE_AUTO = 0, KLEOS_SCHEDULE_DYNAMIC = 1, KLEOS_SCHEDULE_STATIC = 2 };
+int kleos_set_schedule(int schedule);
+int kleos_get_schedule(void);
+/* The schedule the most recent persistent launch took: KLEOS_SCHEDULE_DYNAMIC or
+ * KLEOS_SCHEDULE_STATIC. Synchronises the library stream. KLEOS_ESTATE before the first launch. */
+int kleos_schedule_taken(int* schedule);
+
 /* ---- inspection (no counterpart in the reference, which exposes only gateOut and moeOut) ---- */
 /*
  * Device pointers to the routing state left by the most recent forward, for parity checks of the

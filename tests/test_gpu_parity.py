@@ -38,10 +38,19 @@ def _out_to_np(c, oP):
     return oP.cpu().numpy()
 
 
+def _apply(mode):
+    """mode: a MODE_* value or a (MODE_*, SCHEDULE_*) pair."""
+    if isinstance(mode, tuple):
+        ka.moe.set_mode(mode[0])
+        ka.moe.set_schedule(mode[1])
+    else:
+        ka.moe.set_mode(mode)
+
+
 def run_gpu(keys: ka.KleosConfig, iP_dev, mode, launches=1):
     d = ka.initialize(keys)
     try:
-        ka.moe.set_mode(mode)
+        _apply(mode)
         oP = synth.alloc_outputs(d)
         oP.fill_(float("nan"))           # every output element must be written by the layer
         torch.cuda.synchronize()
@@ -91,8 +100,9 @@ def check_against_oracle(c, keys, iP_np, mode, launches=1, token_mask=None, logi
     return d, v, moe_out, err
 
 
-MODES = [ka.MODE_PHASED, ka.MODE_FUSED]
-MODE_IDS = ["phased", "fused"]
+# (mode, schedule of the persistent launch)
+MODES = [(ka.MODE_PHASED, ka.SCHEDULE_AUTO), (ka.MODE_FUSED, ka.SCHEDULE_DYNAMIC), (ka.MODE_FUSED, ka.SCHEDULE_STATIC)]
+MODE_IDS = ["phased", "fused", "fused-static"]
 
 
 def _keys(S, H, I, E, k, cf=1.0, drop=1, act=0, dt=2):
@@ -232,7 +242,7 @@ def test_new_inputs_in_the_same_context(mode):
     c = moe_ref.cfg_from_keys(keys)
     d = ka.initialize(keys)
     try:
-        ka.moe.set_mode(mode)
+        _apply(mode)
         oP = synth.alloc_outputs(d)
         for seed in (21, 22, 23):
             x, wg, w_up, w_down, *_ = random_layer(c, seed=seed, w_std=0.3 if seed == 22 else 0.08)
@@ -294,9 +304,53 @@ def test_fused_and_phased_agree_bitwise():
     for mode in MODES:
         d, oP, v = run_gpu(keys, iP, mode)
         outs.append((_out_to_np(c, oP), v))
-    np.testing.assert_array_equal(outs[0][0], outs[1][0])
-    for name in ("logits", "topk_expert", "topk_slot", "expert_count"):
-        np.testing.assert_array_equal(outs[0][1][name], outs[1][1][name])
+    for other in outs[1:]:
+        np.testing.assert_array_equal(outs[0][0], other[0])
+        for name in ("logits", "topk_expert", "topk_slot", "expert_count"):
+            np.testing.assert_array_equal(outs[0][1][name], other[1][name])
+
+
+def test_schedule_of_the_persistent_launch():
+    """KLEOS_SCHEDULE_AUTO takes the static schedule when the XCD queues hold equal work and the
+    dynamic one when they do not; a context that alternates between the two (the static schedule
+    holds a grid barrier of its own, whose counters advance only with it) returns the same bits every
+    time, and the same as separate launches per phase."""
+    keys = _keys(2048, 256, 512, 16, 2)
+    c = moe_ref.cfg_from_keys(keys)
+    x, wg, w_up, w_down, *_ = random_layer(c, seed=51, w_std=0.05)
+    balanced = _to_device(c, pack_inputs(c, x, wg, w_up, w_down))
+    # every token to experts 0 and 1: two XCD queues hold all the work
+    wg2 = np.zeros_like(wg)
+    wg2[0, :] = 1.0
+    wg2[1, :] = 0.5
+    skewed = _to_device(c, pack_inputs(c, np.abs(x), wg2, w_up, w_down))
+    _, ref_b, _ = run_gpu(keys, balanced, ka.MODE_PHASED)
+    _, ref_s, _ = run_gpu(keys, skewed, ka.MODE_PHASED)
+    ref_b, ref_s = _out_to_np(c, ref_b), _out_to_np(c, ref_s)
+    d = ka.initialize(keys)
+    try:
+        ka.moe.set_mode(ka.MODE_FUSED)
+        assert ka._capi.lib().kleos_get_schedule() == ka.SCHEDULE_AUTO
+        with pytest.raises(ka.KleosError):
+            ka.moe.set_schedule(7)
+        oP = synth.alloc_outputs(d)
+        plan = [(ka.SCHEDULE_AUTO, balanced, ref_b, ka.SCHEDULE_STATIC),
+                (ka.SCHEDULE_AUTO, skewed, ref_s, ka.SCHEDULE_DYNAMIC),
+                (ka.SCHEDULE_AUTO, balanced, ref_b, ka.SCHEDULE_STATIC),
+                (ka.SCHEDULE_DYNAMIC, balanced, ref_b, ka.SCHEDULE_DYNAMIC),
+                (ka.SCHEDULE_STATIC, skewed, ref_s, ka.SCHEDULE_STATIC),
+                (ka.SCHEDULE_DYNAMIC, skewed, ref_s, ka.SCHEDULE_DYNAMIC),
+                (ka.SCHEDULE_STATIC, balanced, ref_b, ka.SCHEDULE_STATIC),
+                (ka.SCHEDULE_STATIC, balanced, ref_b, ka.SCHEDULE_STATIC)]
+        for step, (schedule, iP, ref, taken) in enumerate(plan):
+            ka.moe.set_schedule(schedule)
+            oP.fill_(float("nan"))
+            torch.cuda.synchronize()
+            ka.moe.forward_host(iP, oP)
+            assert ka.moe.schedule_taken() == taken, f"step {step}"
+            np.testing.assert_array_equal(_out_to_np(c, oP), ref, err_msg=f"step {step}")
+    finally:
+        ka.finalize()
 
 
 # ------------------------------------------------------------------ benchmark-sized configurations
@@ -370,7 +424,7 @@ def test_training_mode_gate_loss(E, k, S):
     for mode in MODES:
         d = ka.initialize(keys)
         try:
-            ka.moe.set_mode(mode)
+            _apply(mode)
             oP = synth.alloc_outputs(d)
             ka.moe.forward_host(iP, oP)
             ka.moe.forward_host(iP, oP)
@@ -378,17 +432,18 @@ def test_training_mode_gate_loss(E, k, S):
             got[mode] = (ka.moe.gate_loss(d.E), ka.moe.debug_views(d), _out_to_np(c, oP))
         finally:
             ka.finalize()
-    g, v, out = got[ka.MODE_FUSED]
+    g, v, out = got[MODES[1]]
     r = moe_ref.route(c, v["logits"])
     np.testing.assert_array_equal(v["expert_count"], r["expert_count"])
     ref = moe_ref.gate_loss(c, r["probs"], r["expert_count"])
     assert abs(g["loss"] - ref["loss"]) < 2e-5 * ref["loss"] + 1e-9, (g["loss"], ref["loss"])
     np.testing.assert_allclose(g["mean_prob"], ref["mean_prob"], rtol=2e-5, atol=1e-8)
     np.testing.assert_allclose(g["mean_count"], ref["mean_count"], rtol=1e-6, atol=0)
-    gp, vp, outp = got[ka.MODE_PHASED]
-    assert gp["loss"] == g["loss"]
-    np.testing.assert_array_equal(gp["mean_prob"], g["mean_prob"])
-    np.testing.assert_array_equal(outp, out)
+    for other in (MODES[0], MODES[2]):
+        gp, vp, outp = got[other]
+        assert gp["loss"] == g["loss"]
+        np.testing.assert_array_equal(gp["mean_prob"], g["mean_prob"])
+        np.testing.assert_array_equal(outp, out)
 
 
 def test_gate_loss_needs_training_mode():
