@@ -63,6 +63,7 @@ struct GemmTileArgs {
     const elem16_t* bias;          // first of the tile's bias entries
     elem16_t* c_base;              // output element (row 0, column 0) of the tile
     uint32_t lda, ldb, ldc, K;
+    uint32_t k_first;              // K slice the tile starts with (it wraps around); below K / BK
     uint32_t m_valid, n_valid;     // rows / columns of the tile that exist
     uint32_t act;                  // 0 relu, 1 erf-gelu, 2 identity
 };
@@ -159,6 +160,7 @@ struct Gemm16 {
     static constexpr int kSmemBytes = STAGES * kStage + 2 * kBiasBytes;
     static constexpr int LA = BM / (kRowsPerLoad * kWaves), LB = BN / (kRowsPerLoad * kWaves);
     static constexpr int kLoadsPerSlice = LA + LB;                 // per wavefront
+    static constexpr int kSliceK = BK;                             // values of K per slice
     static constexpr int kSteps = BK / 16;                         // matrix instructions consume 16 values of K
     static constexpr int kPanelRows = kEpiloguePanelRows;          // epilogue staging: 32 rows x 64 columns per wavefront
     static constexpr int kIssueSteps = kSteps;                     // K steps over which the next slice's loads are issued
@@ -180,7 +182,8 @@ struct Gemm16 {
         const elem16_t* pb[LB];
         elem16_t* c_base;
         uint32_t ldc, m_valid, n_valid, k_tiles, act;
-        int stage0;                 // stage of K slice 0; slice kt uses (stage0 + kt) % STAGES
+        uint32_t k_first;           // the kt-th slice the tile works on is slice (k_first + kt) % k_tiles of K
+        int stage0;                 // stage of the tile's first slice; its kt-th slice uses (stage0 + kt) % STAGES
         int bias_slot;              // which of the two LDS bias slots holds this tile's bias
     };
 
@@ -193,7 +196,9 @@ struct Gemm16 {
         const int wave = threadIdx.x >> 6;
         char* sa = smem + stage_of(t, kt) * kStage;
         char* sb = sa + kABytes;
-        const uint32_t k0 = kt * BK;
+        uint32_t slice = kt + t.k_first;
+        slice = slice >= t.k_tiles ? slice - t.k_tiles : slice;
+        const uint32_t k0 = slice * BK;
 #pragma unroll
         for (int i = 0; i < LA; ++i)
             if (i * parts / LA == part)
@@ -239,6 +244,7 @@ struct Gemm16 {
         }
         t.c_base = g.c_base; t.ldc = g.ldc;
         t.m_valid = g.m_valid; t.n_valid = g.n_valid; t.k_tiles = g.K / BK;
+        t.k_first = g.k_first < t.k_tiles ? g.k_first : 0u;
         t.act = g.act; t.stage0 = stage0; t.bias_slot = bias_slot;
 #pragma unroll
         for (int st = 0; st < STAGES - 1; ++st)
