@@ -142,7 +142,8 @@ __device__ __forceinline__ void epilogue16(const TileOut& t, f32x16 (&acc)[WN / 
     else epilogue16_act<E, WM, WN, WAVES_N, 2>(t, acc, stage_mem, bias_mem);
 }
 
-template <typename E, int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES>
+// ISSUE: over how many K steps of a slice the loads of the slice STAGES-1 ahead are issued.
+template <typename E, int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES, int ISSUE>
 struct Gemm16 {
     typedef typename Elem16<E>::vec8 vec8;
     typedef typename Elem16<E>::vec4 vec4;
@@ -163,7 +164,8 @@ struct Gemm16 {
     static constexpr int kSliceK = BK;                             // values of K per slice
     static constexpr int kSteps = BK / 16;                         // matrix instructions consume 16 values of K
     static constexpr int kPanelRows = kEpiloguePanelRows;          // epilogue staging: 32 rows x 64 columns per wavefront
-    static constexpr int kIssueSteps = kSteps;                     // K steps over which the next slice's loads are issued
+    static constexpr int kIssueSteps = ISSUE;                      // K steps over which the next slice's loads are issued
+    static_assert(ISSUE >= 1 && ISSUE <= kSteps);
     static_assert(BK == 32 || BK == 64);
     static_assert(STAGES >= 2 && STAGES <= 4);
     static_assert(WM % 32 == 0 && WN % 64 == 0);

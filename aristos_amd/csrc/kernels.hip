@@ -29,24 +29,33 @@ constexpr int kXcds = 8;
 // Expert GEMM configuration of the bf16 path: 256 x 256 tile (an expert's whole capacity of 256 rows
 // at the headline shape, so its weights stream from HBM exactly once), 2 x 4 wavefronts of 128 x 64
 // (two per SIMD), K slices of 64 (whole 128-byte lines of every row) through two 64 KB stages.
-// (Measured against it on MI355X, none faster: K slices of 32 through four stages, all loads of a
-// slice issued at its first K step, 2 x 2 wavefronts of 128 x 128 with the accumulators in AGPRs,
-// weight slices of 64 through three slots with activation half slices of 32 through three.)
+// The loads of the next slice are issued over the first two of the four K steps of a slice.
+// (Measured against it on MI355X, none faster: K slices of 32 through four stages, 2 x 2 wavefronts
+// of 128 x 128 with the accumulators in AGPRs, weight slices of 64 through three slots with
+// activation half slices of 32 through three, the 128 x 256 tile of variant 1.)
 // Variant 1, for layers whose experts hold at most 128 rows (many small experts): a 128 x 256 tile
 // wastes no matrix work and no activation loads on rows that do not exist, and its smaller stages
 // leave room for a third one (measured on the 256-expert top-8 shape: 3.7 ms against 4.6 ms).
+// Variant 2, for layers whose experts hold at least four row blocks (few large experts: every
+// weight tile is shared by several workgroups through L2 and loads return quickly): the tile of
+// variant 0 with all loads of the next slice issued at the first K step (measured on the 8-expert
+// top-2 shape with hidden size 4096: 3.8 ms against 3.9 ms with two issue steps and 4.0 with four;
+// at the headline shape, whose weights stream from HBM, one step loses 6 % against two).
 template <typename E, int V>
-using GemmCfg = std::conditional_t<V == 0, Gemm16<E, 256, 256, 2, 4, 64, 2>, Gemm16<E, 128, 256, 2, 4, 64, 3>>;
+using GemmCfg = std::conditional_t<V == 0, Gemm16<E, 256, 256, 2, 4, 64, 2, 2>,
+                std::conditional_t<V == 1, Gemm16<E, 128, 256, 2, 4, 64, 3, 1>, Gemm16<E, 256, 256, 2, 4, 64, 2, 1>>>;
 constexpr int kBN = 256;
 constexpr int kGemmThreads = GemmCfg<bf16_t, 0>::kThreads;
-static_assert(GemmCfg<bf16_t, 1>::kThreads == kGemmThreads, "both variants share the workgroup size");
+static_assert(GemmCfg<bf16_t, 1>::kThreads == kGemmThreads && GemmCfg<bf16_t, 2>::kThreads == kGemmThreads,
+              "all variants share the workgroup size");
 constexpr uint32_t kNarrowRows = 128;   // variant 1 when no expert can hold more rows than this
+constexpr uint32_t kSharedRows = 1024;  // variant 2 when every expert can hold at least this many
 
 // Tile shape and workgroup size of the expert projections per Element type. The workgroup size is
 // also that of the persistent kernel, whose other phases run on groups of its wavefronts.
 template <typename T, int V = 0> struct TileShape {
     static_assert(sizeof(T) == 2);
-    static constexpr int BM = V == 0 ? 256 : 128, BN = kBN, kThreads = kGemmThreads, kPerCu = 1;
+    static constexpr int BM = V == 1 ? 128 : 256, BN = kBN, kThreads = kGemmThreads, kPerCu = 1;
 };
 template <int V> struct TileShape<float, V> { static constexpr int BM = kF32Tile, BN = kF32Tile, kThreads = 256, kPerCu = 1; };
 constexpr int kPhaseThreads = 256;   // gate, slot and combine kernels of the phased mode
@@ -696,6 +705,7 @@ hipError_t dispatch_variant(const LayerParams& p, F&& f) {
     if constexpr (sizeof(T) == 2) {
         const uint32_t cap = p.EC < p.cap_rows ? p.EC : p.cap_rows;
         if (cap <= kNarrowRows) return f(std::integral_constant<int, 1>{});
+        if (cap >= kSharedRows) return f(std::integral_constant<int, 2>{});
     }
     return f(std::integral_constant<int, 0>{});
 }

@@ -150,6 +150,7 @@ CASES = [
     (256, 128, 256, 8, 2, 1.0, 1, 0, 3, 0.0),      # fp16
     (256, 192, 320, 12, 3, 1.0, 1, 1, 3, 0.1),     # fp16, gelu + biases, ragged sizes
     (512, 256, 256, 64, 2, 1.0, 1, 0, 3, 0.0),     # fp16, E = 64, several K slices
+    (2048, 192, 320, 2, 2, 1.0, 1, 1, 2, 0.1),     # 2048 rows per expert: the tile variant of large experts
 ]
 
 
