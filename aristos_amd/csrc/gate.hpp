@@ -30,9 +30,9 @@ template <int NG>
 constexpr int gate_unit_blocks() { return NG >= 16 ? 1 : 2; }
 
 // LDS floats needed by gate_unit with KW wavefronts: the partial accumulators (4*NG registers of
-// 64 lanes) of the KW-1 wavefronts that do not own the block being reduced.
+// 64 lanes) of the KW shares of the hidden dimension of the block being reduced.
 template <int NG>
-constexpr int gate_smem_floats(int kw) { return (kw - 1) * NG * 4 * kWave; }
+constexpr int gate_smem_floats(int kw) { return kw * NG * 4 * kWave; }
 
 // Softmax, top-k, outputs and the tile histogram of one 16-token tile, run by one wavefront that
 // holds the complete logits of the tile: acc[g][v] of lane l is expert 16 g + 4 (l / 16) + v of
@@ -192,7 +192,11 @@ __device__ __forceinline__ void gate_unit(const LayerParams& p, uint32_t unit, f
     constexpr int kStepK = GateK<T>::kStepK;
     constexpr int kPer = GateK<T>::kElemsPer16B;
     const uint32_t steps = H / kStepK;
-    const uint32_t s0 = (steps * wave) / KW, s1 = (steps * (wave + 1)) / KW;
+    // Wavefront w works on share (w + unit / 8) % KW of the hidden dimension: the units that run on
+    // one XCD at the same time (unit numbers 8 apart) then ask its L2 for different lines of the
+    // gate weights at any moment instead of all for the same ones.
+    const uint32_t part = (uint32_t(wave) + (unit >> 3)) % uint32_t(KW);
+    const uint32_t s0 = (steps * part) / KW, s1 = (steps * (part + 1)) / KW;
 
     const T* xrow[TB];
     bool live[TB];
@@ -249,21 +253,24 @@ __device__ __forceinline__ void gate_unit(const LayerParams& p, uint32_t unit, f
         }
     }
 
-    // Block b: every wavefront but b parks its partial sums in LDS, wavefront b adds them to its
-    // own in ascending wavefront order (a fixed order: the logits do not depend on timing).
+    // Block b: every wavefront parks the partial sums of its share in LDS, wavefront b adds them
+    // in ascending order of the shares (a fixed order: the logits depend neither on timing nor on
+    // which wavefront worked on which share).
 #pragma unroll
     for (int b = 0; b < TB; ++b) {
-        if (wave != b) {
-            float* dst = smem + (wave - (wave > b ? 1 : 0)) * (NG * 4 * kWave);
+        float* dst = smem + part * (NG * 4 * kWave);
 #pragma unroll
-            for (int g = 0; g < NG; ++g)
+        for (int g = 0; g < NG; ++g)
 #pragma unroll
-                for (int v = 0; v < 4; ++v) dst[(g * 4 + v) * kWave + lane] = acc[b][g][v];
-        }
+            for (int v = 0; v < 4; ++v) dst[(g * 4 + v) * kWave + lane] = acc[b][g][v];
         __syncthreads();
         if (wave == b) {
 #pragma unroll
-            for (int w = 0; w < KW - 1; ++w) {
+            for (int g = 0; g < NG; ++g)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) acc[b][g][v] = smem[(g * 4 + v) * kWave + lane];
+#pragma unroll
+            for (int w = 1; w < KW; ++w) {
                 const float* src = smem + w * (NG * 4 * kWave);
 #pragma unroll
                 for (int g = 0; g < NG; ++g)
