@@ -26,7 +26,7 @@ PEAK_HBM_GBS = 8000.0
 # WRITE_SIZE, each scaled by what the counter reads for a 1 GiB copy) summarised in
 # profiles/fused_kernel_headline_e64_zipf_hbm_traffic.txt. Counters cannot be read inside a timed
 # run, so the figure is carried here; --traffic-bytes overrides it after a new pair of passes.
-MEASURED_TRAFFIC_BYTES = {"headline_e64_zipf": 1.4174e9}
+MEASURED_TRAFFIC_BYTES = {"headline_e64_zipf": 1.4330e9}
 
 
 def main() -> int:
@@ -93,6 +93,7 @@ def main() -> int:
         ev_ms = ka.moe.forward_host_bench(iP, oP, skip=0, trials=args.steps)
         fused_ph = ka.moe.phase_times()
         sched = ka.moe.scheduler_stats()
+        schedule = "static" if ka.moe.schedule_taken() == ka.SCHEDULE_STATIC else "dynamic"
         views = ka.moe.debug_views(d)
         kept = int(np.minimum(views["expert_count"].astype(np.int64), d.kept_capacity).sum())
         dropped = int((views["topk_slot"] < 0).sum())
@@ -152,7 +153,8 @@ def main() -> int:
         "config": {"workload": f"{w.name}: {w.note}", "S": d.S, "H": d.H, "I": d.I, "E": d.E, "top_k": d.k,
                    "capacity_factor": w.config.capacity_factor, "EC": d.EC, "kept_pairs": kept,
                    "dropped_pairs": dropped, "hottest_expert_vs_mean": round(hottest, 2),
-                   "mode": "fused persistent kernel, 1 launch per forward"},
+                   "mode": "fused persistent kernel, 1 launch per forward",
+                   "expert_schedule": schedule + " (KLEOS_SCHEDULE_AUTO)"},
         "tokens_per_s": round(d.S / (wall_ms * 1e-3), 1),
         "event_ms_per_step": round(ev_ms, 5),
         "roofline": roofline(flops_layer, hbm_bytes, ev_ms, peak, args.traffic_bytes),
