@@ -133,12 +133,18 @@ __device__ __forceinline__ void bounded_wait(uint32_t* sched, Pred&& pred) {
 // each counter instead of one per workgroup on a single word, which is what a flat barrier spends
 // most of its time on when everybody arrives together. All counters only ever grow, so nothing is
 // reset between launches.
-__device__ __forceinline__ void grid_barrier(uint32_t* sched, uint32_t which, uint32_t seq, uint32_t nwg) {
+// `between()` is called by every thread after the workgroup has arrived and before it waits for the
+// others: work that does not depend on what the other workgroups are still writing rides in the
+// wait. The arrival and the wait are the business of the first lane of the last wavefront, so that
+// the wavefronts `between` keeps busy (it may hold workgroup barriers) do not sit behind the
+// arrival's trips to memory longer than they must.
+template <typename Between>
+__device__ __forceinline__ void grid_barrier(uint32_t* sched, uint32_t which, uint32_t seq, uint32_t nwg, Between&& between) {
     __syncthreads();
-    if (threadIdx.x == 0) {
+    const bool leader = threadIdx.x == blockDim.x - kWave;
+    if (leader) {
         const uint32_t g = blockIdx.x % kXcds;
         const uint32_t members = (nwg - g + kXcds - 1) / kXcds;
-        const uint32_t groups = nwg < uint32_t(kXcds) ? nwg : uint32_t(kXcds);
         uint32_t* all = sched + kSchedBar + which * kSchedLine;
         uint32_t* mine = sched + kSchedGroup + (which * kXcds + g) * kSchedLine;
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
@@ -146,6 +152,11 @@ __device__ __forceinline__ void grid_barrier(uint32_t* sched, uint32_t which, ui
             __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "agent");
             atomic_add_agent(all, 1u);
         }
+    }
+    between();
+    if (leader) {
+        const uint32_t groups = nwg < uint32_t(kXcds) ? nwg : uint32_t(kXcds);
+        uint32_t* all = sched + kSchedBar + which * kSchedLine;
         const uint32_t target = (seq + 1u) * groups;
         bounded_wait(sched, [&] { return int32_t(atomic_load_relaxed(all) - target) >= 0; });
     }
@@ -154,6 +165,27 @@ __device__ __forceinline__ void grid_barrier(uint32_t* sched, uint32_t which, ui
     // microseconds of refetching per launch). What crosses workgroups after a barrier is read
     // with device-coherent loads instead; this only drops the CU's own L1.
     asm volatile("buffer_inv sc0" ::: "memory");
+}
+
+__device__ __forceinline__ void grid_barrier(uint32_t* sched, uint32_t which, uint32_t seq, uint32_t nwg) {
+    grid_barrier(sched, which, seq, nwg, [] {});
+}
+
+// Tokens the gate routed to expert e in this launch, dropped ones included: the sum of the coarse
+// count rows, which are complete once the gate phase has been released.
+__device__ __forceinline__ uint32_t routed_count(const LayerParams& p, uint32_t e) {
+    const uint32_t* super = p.super_count + size_t(p.epoch & 1u) * p.n_super * p.E;
+    uint32_t total = 0;
+    constexpr uint32_t kBatch = 16;
+    for (uint32_t r0 = 0; r0 < p.n_super; r0 += kBatch) {
+        uint32_t v[kBatch];
+#pragma unroll
+        for (uint32_t u = 0; u < kBatch; ++u)
+            v[u] = load_coherent(super + size_t(r0 + u < p.n_super ? r0 + u : p.n_super - 1) * p.E + e);
+#pragma unroll
+        for (uint32_t u = 0; u < kBatch; ++u) total += r0 + u < p.n_super ? v[u] : 0u;
+    }
+    return total;
 }
 
 // Barrier among the `members` workgroups that run on XCD `xcd`, the `runs`-th time it is held on this
@@ -503,8 +535,6 @@ __global__ __launch_bounds__((TileShape<T, V>::kThreads), (TileShape<T, V>::kPer
         for (uint32_t i = blockIdx.x * kThreads + tid; i < p.n_super * p.E; i += nwg * kThreads) other[i] = 0u;
     }
     if (tid == 0) stamp[3] = wall_clock64();
-    grid_barrier(sched, 1, seq, nwg);
-    if (tid == 0) stamp[4] = wall_clock64();
 
     // ---- phase 2: expert tiles from per-XCD ticket queues
     // LDS map: row blocks per expert | queue starts, totals, task | segments | GEMM tile
@@ -524,82 +554,89 @@ __global__ __launch_bounds__((TileShape<T, V>::kThreads), (TileShape<T, V>::kPer
     char* s_gemm = smem + kFusedLdsHeader;
     const uint32_t tn_up = ceil_div_u32(p.I, BN), tn_down = ceil_div_u32(p.H, BN);
 
-    // how many workgroups every XCD holds: asked for first, so that the answers travel together
-    // with the routed counts below
-    uint32_t seen[kXcds] = {};
-    if (tid == 0)
-        for (uint32_t j = 0; j < kXcds; ++j) seen[j] = atomic_load_relaxed(members_now + j * kSchedLine);
-    for (uint32_t e = tid; e < p.E; e += kThreads) {
-        const uint32_t rows = kept_rows<true>(p, e);
-        s_rows[e] = rows;
-        s_mt[e] = uint16_t(ceil_div_u32(rows, BM));
-    }
-    __syncthreads();
+    // The queues of the expert phase are set up while this workgroup waits for the others to finish
+    // the slot phase: what the set-up reads (the routed counts the gate accumulated, the workgroups
+    // per XCD) has been complete since the first barrier.
     const uint32_t members = nwg / kXcds;
-    // Static or dynamic schedule: every workgroup decides alike, from the same counters.
-    // Static: each XCD's workgroups stride through their queue's up tiles, meet at a barrier, then
-    // stride through its down tiles: no tickets, no readiness counters, no per-tile publication.
-    // It needs every XCD to hold the same number of workgroups, and it pays only when the queues
-    // hold about the same work (nobody to steal from).
-    // Thread q sets up queue q; its segments start at a fixed place, two per expert of the queue.
-    const uint32_t my_nq = tid < p.E && tid < uint32_t(kXcds) ? (p.E - tid + kXcds - 1) / kXcds : 0u;   // experts q, q+8, ...
-    if (tid < uint32_t(kXcds)) {
-        uint32_t blocks = 0;
-        for (uint32_t i = 0; i < my_nq; ++i) blocks += s_mt[tid + kXcds * i];
-        s_qtot[tid] = blocks;
-    }
-    if (tid == 0) {
-        bool even = nwg % kXcds == 0;
-        for (uint32_t j = 0; j < kXcds; ++j) even = even && seen[j] == members;
-        s_static[1] = my_rank;
-        s_static[2] = static_runs;
-        s_static[3] = my_rank;
-        s_static[4] = 0u;
-        s_static[5] = even;
-    }
-    __syncthreads();
-    bool use_static;
-    {
-        uint32_t lo = ~0u, hi = 0;
-        for (uint32_t q = 0; q < kXcds; ++q) {
-            const uint32_t blocks = s_qtot[q];
-            lo = blocks < lo ? blocks : lo;
-            hi = blocks > hi ? blocks : hi;
+    bool use_static = false;
+    grid_barrier(sched, 1, seq, nwg, [&] {
+        // how many workgroups every XCD holds: asked for first, so that the answers travel together
+        // with the routed counts below
+        uint32_t seen[kXcds] = {};
+        if (tid == 0)
+            for (uint32_t j = 0; j < kXcds; ++j) seen[j] = atomic_load_relaxed(members_now + j * kSchedLine);
+        for (uint32_t e = tid; e < p.E; e += kThreads) {
+            const uint32_t routed = routed_count(p, e);
+            const uint32_t cap = p.EC < p.cap_rows ? p.EC : p.cap_rows;
+            const uint32_t rows = routed < cap ? routed : cap;   // consumers clamp the routed count to the capacity (packet.cuh:85,112-113)
+            s_rows[e] = rows;
+            s_mt[e] = uint16_t(ceil_div_u32(rows, BM));
         }
-        const bool balanced = hi - lo <= hi / 16;
-        // the same in every lane: keep it in a scalar register
-        use_static = __builtin_amdgcn_readfirstlane(int(s_static[5] != 0 && balanced_or_forced(policy, balanced))) != 0;
-    }
-    __syncthreads();   // the row-block sums above shared s_qtot with the ticket totals below
-    if (tid < uint32_t(kXcds)) {
-        const uint32_t q = tid, nq = my_nq;
-        const uint32_t first = 2 * (q * (p.E / kXcds) + (q < p.E % kXcds ? q : p.E % kXcds));
-        uint32_t nseg = first;
-        s_qseg[q] = first;
-        if (q == kXcds - 1) s_qseg[kXcds] = 2 * p.E;
-        const uint32_t lag = use_static ? nq : dynamic_lag;   // static: all ups, then all downs
-        uint32_t ticket = 0, ups = 0;
-        // up-projection of expert i, then down-projection of expert i - lag: a down tile is
-        // handed out only after `lag` further experts' worth of tickets, by which time the
-        // up tiles it depends on have normally been stored.
-        for (uint32_t i = 0; i < nq + lag; ++i) {
-            if (i < nq) {
-                const uint32_t e = q + kXcds * i;
-                s_seg[nseg++] = Segment{uint16_t(e), 0, 0, ticket};
-                ticket += uint32_t(s_mt[e]) * tn_up;
-                ups += uint32_t(s_mt[e]) * tn_up;
-            }
-            if (i >= lag && i - lag < nq) {
-                const uint32_t e = q + kXcds * (i - lag);
-                s_seg[nseg++] = Segment{uint16_t(e), 1, 0, ticket};
-                ticket += uint32_t(s_mt[e]) * tn_down;
-            }
+        __syncthreads();
+        // Static or dynamic schedule: every workgroup decides alike, from the same counters.
+        // Static: each XCD's workgroups stride through their queue's up tiles, meet at a barrier, then
+        // stride through its down tiles: no tickets, no readiness counters, no per-tile publication.
+        // It needs every XCD to hold the same number of workgroups, and it pays only when the queues
+        // hold about the same work (nobody to steal from).
+        // Thread q sets up queue q; its segments start at a fixed place, two per expert of the queue.
+        const uint32_t my_nq = tid < p.E && tid < uint32_t(kXcds) ? (p.E - tid + kXcds - 1) / kXcds : 0u;   // experts q, q+8, ...
+        if (tid < uint32_t(kXcds)) {
+            uint32_t blocks = 0;
+            for (uint32_t i = 0; i < my_nq; ++i) blocks += s_mt[tid + kXcds * i];
+            s_qtot[tid] = blocks;
         }
-        s_qtot[q] = ticket;
-        s_qup[q] = ups;
-    }
-    __syncthreads();
-    if (tid == 0) stamp[14] = use_static;
+        if (tid == 0) {
+            bool even = nwg % kXcds == 0;
+            for (uint32_t j = 0; j < kXcds; ++j) even = even && seen[j] == members;
+            s_static[1] = my_rank;
+            s_static[2] = static_runs;
+            s_static[3] = my_rank;
+            s_static[4] = 0u;
+            s_static[5] = even;
+        }
+        __syncthreads();
+        {
+            uint32_t lo = ~0u, hi = 0;
+            for (uint32_t q = 0; q < kXcds; ++q) {
+                const uint32_t blocks = s_qtot[q];
+                lo = blocks < lo ? blocks : lo;
+                hi = blocks > hi ? blocks : hi;
+            }
+            const bool balanced = hi - lo <= hi / 16;
+            // the same in every lane: keep it in a scalar register
+            use_static = __builtin_amdgcn_readfirstlane(int(s_static[5] != 0 && balanced_or_forced(policy, balanced))) != 0;
+        }
+        __syncthreads();   // the row-block sums above shared s_qtot with the ticket totals below
+        if (tid < uint32_t(kXcds)) {
+            const uint32_t q = tid, nq = my_nq;
+            const uint32_t first = 2 * (q * (p.E / kXcds) + (q < p.E % kXcds ? q : p.E % kXcds));
+            uint32_t nseg = first;
+            s_qseg[q] = first;
+            if (q == kXcds - 1) s_qseg[kXcds] = 2 * p.E;
+            const uint32_t lag = use_static ? nq : dynamic_lag;   // static: all ups, then all downs
+            uint32_t ticket = 0, ups = 0;
+            // up-projection of expert i, then down-projection of expert i - lag: a down tile is
+            // handed out only after `lag` further experts' worth of tickets, by which time the
+            // up tiles it depends on have normally been stored.
+            for (uint32_t i = 0; i < nq + lag; ++i) {
+                if (i < nq) {
+                    const uint32_t e = q + kXcds * i;
+                    s_seg[nseg++] = Segment{uint16_t(e), 0, 0, ticket};
+                    ticket += uint32_t(s_mt[e]) * tn_up;
+                    ups += uint32_t(s_mt[e]) * tn_up;
+                }
+                if (i >= lag && i - lag < nq) {
+                    const uint32_t e = q + kXcds * (i - lag);
+                    s_seg[nseg++] = Segment{uint16_t(e), 1, 0, ticket};
+                    ticket += uint32_t(s_mt[e]) * tn_down;
+                }
+            }
+            s_qtot[q] = ticket;
+            s_qup[q] = ups;
+        }
+        __syncthreads();
+    });
+    if (tid == 0) { stamp[4] = wall_clock64(); stamp[14] = use_static; }
 
     uint32_t q_off = 0;   // queues already found empty, starting from this workgroup's own XCD
     uint32_t q_dead = 0;  // bit q: queue q was seen exhausted
