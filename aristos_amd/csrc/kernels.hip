@@ -11,6 +11,9 @@
 //     a statically ordered tile list, and one readiness counter per (expert, row block) that
 //     releases the down-projection tiles once all up-projection tiles of that block are stored
 //     (the reference's tQS counter + notifyNext, os/processor/processor.cuh:516-636,719-729).
+//     When the queues hold equal work the same tile list is walked without tickets: each XCD's
+//     workgroups stride through it by a rank they take at the start, with one barrier among them
+//     between the projections (the static schedule, chosen per launch inside the kernel).
 #include "kernels.hpp"
 
 #include <type_traits>
@@ -536,7 +539,7 @@ __global__ __launch_bounds__((TileShape<T, V>::kThreads), (TileShape<T, V>::kPer
     }
     if (tid == 0) stamp[3] = wall_clock64();
 
-    // ---- phase 2: expert tiles from per-XCD ticket queues
+    // ---- phase 2: expert tiles from the per-XCD queues (by ticket, or by stride in the static schedule)
     // LDS map: row blocks per expert | queue starts, totals, task | segments | GEMM tile
     uint32_t* s_rows = reinterpret_cast<uint32_t*>(smem);                       // [E], E <= 256: rows kept
     uint16_t* s_mt = reinterpret_cast<uint16_t*>(smem + 1024);                  // [E] row blocks
