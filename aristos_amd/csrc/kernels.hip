@@ -579,8 +579,8 @@ __global__ __launch_bounds__((TileShape<T, V>::kThreads), (TileShape<T, V>::kPer
         // Static or dynamic schedule: every workgroup decides alike, from the same counters.
         // Static: each XCD's workgroups stride through their queue's up tiles, meet at a barrier, then
         // stride through its down tiles: no tickets, no readiness counters, no per-tile publication.
-        // It needs every XCD to hold the same number of workgroups, and it pays only when the queues
-        // hold about the same work (nobody to steal from).
+        // It needs every XCD to hold the same number of workgroups, and it pays only when no queue
+        // would keep its XCD busy for longer than freely handed-out tiles keep the grid busy.
         // Thread q sets up queue q; its segments start at a fixed place, two per expert of the queue.
         const uint32_t my_nq = tid < p.E && tid < uint32_t(kXcds) ? (p.E - tid + kXcds - 1) / kXcds : 0u;   // experts q, q+8, ...
         if (tid < uint32_t(kXcds)) {
@@ -599,13 +599,18 @@ __global__ __launch_bounds__((TileShape<T, V>::kThreads), (TileShape<T, V>::kPer
         }
         __syncthreads();
         {
-            uint32_t lo = ~0u, hi = 0;
+            // rounds = tiles one workgroup works through in a projection. Strided, an XCD needs
+            // ceil(its tiles / its workgroups); handed out freely, the grid needs at least
+            // ceil(all tiles / all workgroups). Static loses nothing when no XCD needs more.
+            uint32_t hi = 0, sum = 0;
             for (uint32_t q = 0; q < kXcds; ++q) {
                 const uint32_t blocks = s_qtot[q];
-                lo = blocks < lo ? blocks : lo;
                 hi = blocks > hi ? blocks : hi;
+                sum += blocks;
             }
-            const bool balanced = hi - lo <= hi / 16;
+            const uint32_t m = members ? members : 1u;
+            const bool balanced = ceil_div_u32(hi * tn_up, m) <= ceil_div_u32(sum * tn_up, m * kXcds) &&
+                                  ceil_div_u32(hi * tn_down, m) <= ceil_div_u32(sum * tn_down, m * kXcds);
             // the same in every lane: keep it in a scalar register
             use_static = __builtin_amdgcn_readfirstlane(int(s_static[5] != 0 && balanced_or_forced(policy, balanced))) != 0;
         }

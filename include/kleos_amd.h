@@ -144,7 +144,8 @@ int kleos_get_mode(void);
  * up-projection tiles of their queue, the grid meets at a barrier, and they stride through the
  * down-projection tiles. It spends nothing per tile on tickets and publication, and loses when the
  * queues hold unequal work. KLEOS_SCHEDULE_AUTO (default) decides inside the kernel, from the
- * routed counts of the launch: static when the row blocks per queue differ by at most 1/16.
+ * routed counts of the launch: static when no XCD's queue takes its workgroups more rounds of tiles
+ * than the whole tile list would take spread over all workgroups.
  * KLEOS_SCHEDULE_STATIC still falls back to the dynamic schedule when the hardware did not place
  * the same number of workgroups on every XCD. Outputs are identical under every schedule. */
 enum { KLEOS_SCHEDULE_AUTO = 0, KLEOS_SCHEDULE_DYNAMIC = 1, KLEOS_SCHEDULE_STATIC = 2 };

@@ -312,15 +312,16 @@ def test_fused_and_phased_agree_bitwise():
 
 
 def test_schedule_of_the_persistent_launch():
-    """KLEOS_SCHEDULE_AUTO takes the static schedule when the XCD queues hold equal work and the
-    dynamic one when they do not; a context that alternates between the two (the static schedule
+    """KLEOS_SCHEDULE_AUTO takes the static schedule when striding through the XCD queues costs no
+    extra round of tiles and the dynamic one when it would; a context that alternates between the two (the static schedule
     holds a grid barrier of its own, whose counters advance only with it) returns the same bits every
     time, and the same as separate launches per phase."""
-    keys = _keys(2048, 256, 512, 16, 2)
+    keys = _keys(8192, 128, 512, 8, 2, cf=8.0)
     c = moe_ref.cfg_from_keys(keys)
     x, wg, w_up, w_down, *_ = random_layer(c, seed=51, w_std=0.05)
     balanced = _to_device(c, pack_inputs(c, x, wg, w_up, w_down))
-    # every token to experts 0 and 1: two XCD queues hold all the work
+    # every token to experts 0 and 1, nothing dropped: two XCD queues hold 64 tiles each per
+    # projection, two rounds for their XCDs' 32 workgroups, one round if the grid shares them
     wg2 = np.zeros_like(wg)
     wg2[0, :] = 1.0
     wg2[1, :] = 0.5
