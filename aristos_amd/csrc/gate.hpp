@@ -6,7 +6,8 @@
 //   * one wavefront quad of lanes owns a token, so softmax and top-k are register + cross-lane
 //     shuffle work; the reference bounces the accumulator through shared memory to get one
 //     thread per token (gate.cuh:560-572);
-//   * every expert count up to 256 is handled inside one workgroup (the reference chains
+//   * every expert count is handled inside one workgroup: up to 256 experts with the logits in
+//     registers, more in passes of 256 with the logits read back from memory (the reference chains
 //     64-expert blocks through global-memory mailboxes, gate.cuh:93-468);
 //   * slots are assigned in token order from per-tile histograms and their prefix sums, which
 //     makes dropping deterministic; the reference takes a tile's base slot from atomicAdd arrival
@@ -26,13 +27,15 @@ struct GateK {
 // Token blocks (16 tokens each) one gate unit works on together: the fragments of the gate weights
 // are loaded once per unit and used by every block, which halves the L2 traffic of the weights.
 // With 16 expert groups (E > 128) the accumulators of two blocks no longer fit the register file.
+// NG = 0 stands for the wide gate (E > 256), which works in passes of 16 groups.
 template <int NG>
-constexpr int gate_unit_blocks() { return NG >= 16 ? 1 : 2; }
+constexpr int gate_unit_blocks() { return NG == 0 || NG >= 16 ? 1 : 2; }
 
 // LDS floats needed by gate_unit with KW wavefronts: the partial accumulators (4*NG registers of
 // 64 lanes) of the KW shares of the hidden dimension of the block being reduced.
 template <int NG>
-constexpr int gate_smem_floats(int kw) { return kw * NG * 4 * kWave; }
+constexpr int gate_smem_floats(int kw) { return kw * (NG == 0 ? 16 : NG) * 4 * kWave; }
+constexpr uint32_t kWideGateMaxK = 32;   // the wide gate keeps a tile's 16 * k picks in LDS
 
 // Softmax, top-k, outputs and the tile histogram of one 16-token tile, run by one wavefront that
 // holds the complete logits of the tile: acc[g][v] of lane l is expert 16 g + 4 (l / 16) + v of
@@ -283,6 +286,176 @@ __device__ __forceinline__ void gate_unit(const LayerParams& p, uint32_t unit, f
 #pragma unroll
     for (int b = 0; b < TB; ++b)
         if (wave == b && live[b]) gate_epilogue<T, NG>(p, unit * TB + b, acc[b], lane);
+    __syncthreads();
+}
+
+// The gate for more than 256 experts: one 16-token block per unit, the experts in passes of 256.
+// Every pass is the K loop and the reduction of gate_unit with 16 groups; wavefront 0 stores the
+// pass's logits, and when all passes are done it reads them back for softmax and top-k (each lane
+// reads exactly the words it stored). Selection needs no record of what was picked: round r takes
+// the largest logit that comes after the previous pick in the order (logit descending, expert
+// ascending), which is the same k rounds of arg-max with ties to the lower index
+// (gate.cuh:654-670). The tile's picks go through LDS for the in-tile ranks and the histogram.
+// Every thread of the workgroup must call the function; `smem` holds gate_smem_floats<0>(KW) floats.
+template <typename T, int KW>
+__device__ __forceinline__ void gate_unit_wide(const LayerParams& p, uint32_t unit, float* smem) {
+    constexpr int NG = 16;
+    const int wave = __builtin_amdgcn_readfirstlane(int(threadIdx.x >> 6)), lane = threadIdx.x & 63;
+    const int col = lane & 15, chunk = lane >> 4;
+    const uint32_t H = p.H, E = p.E, k = p.k;
+    constexpr int kStepK = GateK<T>::kStepK;
+    constexpr int kPer = GateK<T>::kElemsPer16B;
+    const uint32_t steps = H / kStepK;
+    const uint32_t part = (uint32_t(wave) + (unit >> 3)) % uint32_t(KW);
+    const uint32_t s0 = (steps * part) / KW, s1 = (steps * (part + 1)) / KW;
+    const uint32_t tile = unit;
+    const bool live = tile < p.n_gate_tiles;
+    const uint32_t token = (live ? tile : p.n_gate_tiles - 1) * kGateTileTokens + col;
+    const T* xrow = static_cast<const T*>(p.x) + size_t(token) * H + chunk * kPer;
+    float* my_logits = p.logits + size_t(token) * E;
+
+    for (uint32_t e0 = 0; e0 < E; e0 += 16 * NG) {
+        f32x4 acc[NG];
+#pragma unroll
+        for (int g = 0; g < NG; ++g) acc[g] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (uint32_t s = s0; s < s1; ++s) {
+            const uint32_t off = s * kStepK;
+            const u32x4 xb = load16(xrow + off);
+#pragma unroll
+            for (int g = 0; g < NG; ++g) {
+                // weight rows past the padded expert count re-read its last row; their logits are never stored
+                const uint32_t r = e0 + 16 * g + col;
+                const T* wrow = static_cast<const T*>(p.wg) + size_t(r < p.PX ? r : p.PX - 1) * H + chunk * kPer;
+                acc[g] = mma16_step(load16(wrow + off), xb, acc[g], T{});
+            }
+        }
+        float* dst = smem + part * (NG * 4 * kWave);
+#pragma unroll
+        for (int g = 0; g < NG; ++g)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) dst[(g * 4 + v) * kWave + lane] = acc[g][v];
+        __syncthreads();
+        if (wave == 0 && live) {
+#pragma unroll
+            for (int g = 0; g < NG; ++g)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    float sum = smem[(g * 4 + v) * kWave + lane];
+#pragma unroll
+                    for (int w = 1; w < KW; ++w) sum += smem[w * (NG * 4 * kWave) + (g * 4 + v) * kWave + lane];
+                    const uint32_t e = e0 + 16 * g + 4 * chunk + v;
+                    if (e < E) my_logits[e] = sum;
+                }
+        }
+        __syncthreads();
+    }
+
+    if (wave == 0 && live) {
+        // lane (col, chunk) owns experts 16 j + 4 chunk + v of token col, as in the register gate
+        const float kNegInf = -__builtin_inff();
+        const uint32_t groups = (E + 15) / 16;
+        auto logit = [&](uint32_t e) { return load_coherent(my_logits + e); };
+        float m = kNegInf;
+        for (uint32_t j = 0; j < groups; ++j)
+#pragma unroll
+            for (uint32_t v = 0; v < 4; ++v) {
+                const uint32_t e = 16 * j + 4 * chunk + v;
+                if (e < E) m = fmaxf(m, logit(e));
+            }
+        m = fmaxf(m, __shfl_xor(m, 16));
+        m = fmaxf(m, __shfl_xor(m, 32));
+        float d = 0.f;
+        for (uint32_t j = 0; j < groups; ++j)
+#pragma unroll
+            for (uint32_t v = 0; v < 4; ++v) {
+                const uint32_t e = 16 * j + 4 * chunk + v;
+                if (e < E) d += __expf(logit(e) - m);
+            }
+        d += __shfl_xor(d, 16);
+        d += __shfl_xor(d, 32);
+        const float inv_d = 1.0f / d;
+        auto prob = [&](float l) { return __expf(l - m) * inv_d; };
+        T* grow = static_cast<T*>(p.gate_out) + size_t(token) * p.PX;
+        for (uint32_t j = 0; 16 * j < p.PX; ++j)
+#pragma unroll
+            for (uint32_t v = 0; v < 4; ++v) {
+                const uint32_t e = 16 * j + 4 * chunk + v;
+                const float pe = e < E ? prob(logit(e)) : 0.f;
+                if (e < p.PX) grow[e] = float_to_elem<T>(pe);   // padded columns are zero (gate.cuh:590-605)
+                if (p.is_training) {
+                    // column sum over the tile's 16 tokens, a fixed xor tree (gate.cuh:608-635)
+                    float col_sum = pe;
+                    col_sum += __shfl_xor(col_sum, 1);
+                    col_sum += __shfl_xor(col_sum, 2);
+                    col_sum += __shfl_xor(col_sum, 4);
+                    col_sum += __shfl_xor(col_sum, 8);
+                    if (col == 0 && e < E) p.tile_prob[size_t(tile) * E + e] = col_sum;
+                }
+            }
+
+        uint32_t* s_hist = reinterpret_cast<uint32_t*>(smem);   // [E] tokens of the tile routed to e
+        uint32_t* s_sel = s_hist + E;                           // [16][k] the tile's picks
+        for (uint32_t e = lane; e < E; e += kWave) s_hist[e] = 0u;
+        constexpr uint32_t kNone = 0x7fffffffu;
+        float den = 0.f, prev_l = 0.f;
+        uint32_t prev_e = 0;
+        for (uint32_t r = 0; r < k; ++r) {
+            float best = kNegInf;
+            uint32_t bi = kNone;
+            for (uint32_t j = 0; j < groups; ++j)
+#pragma unroll
+                for (uint32_t v = 0; v < 4; ++v) {
+                    const uint32_t e = 16 * j + 4 * chunk + v;
+                    if (e >= E) continue;
+                    const float l = logit(e);
+                    const bool open = r == 0 || l < prev_l || (l == prev_l && e > prev_e);
+                    if (open && (bi == kNone || l > best)) {
+                        best = l;
+                        bi = e;
+                    }
+                }
+#pragma unroll
+            for (int off = 16; off <= 32; off <<= 1) {
+                const float ob = __shfl_xor(best, off);
+                const uint32_t oi = __shfl_xor(bi, off);
+                if (oi != kNone && (bi == kNone || ob > best || (ob == best && oi < bi))) {
+                    best = ob;
+                    bi = oi;
+                }
+            }
+            // all four lanes of the token hold the pick now
+            const float pv = bi != kNone ? prob(best) : 0.f;
+            den += pv;   // mCw, accumulated in selection order (gate.cuh:669)
+            prev_l = best;
+            prev_e = bi;
+            if (chunk == 0) {
+                p.topk_expert[size_t(token) * k + r] = int32_t(bi);
+                p.topk_prob[size_t(token) * k + r] = pv;
+                s_sel[uint32_t(col) * k + r] = bi;
+            }
+        }
+        if (chunk == 0) p.combine_den[token] = den;
+        // in-tile rank of every pick and the tile histogram (gate.cuh:678-696); the LDS operations of
+        // one wavefront complete in order, so the picks written above are visible here
+        uint32_t* super = p.super_count + size_t(p.epoch & 1u) * p.n_super * E + size_t(tile / kSuperTiles) * E;
+        const uint32_t pairs = kGateTileTokens * k;
+        for (uint32_t i = lane; i < pairs; i += kWave) {
+            const uint32_t t = i / k, e = s_sel[i];
+            uint32_t before = 0, total = 0;
+            for (uint32_t o = 0; o < pairs; ++o) {
+                const bool same = s_sel[o] == e;
+                total += same;
+                before += same && o / k < t;
+            }
+            p.topk_slot[(size_t(tile) * kGateTileTokens + t) * k + (i % k)] = int32_t(before);
+            if (before == 0 && e < E) s_hist[e] = total;   // one writer: the first token that picked e
+        }
+        for (uint32_t e = lane; e < E; e += kWave) {
+            const uint32_t cnt = s_hist[e];
+            p.tile_count[size_t(tile) * E + e] = cnt;
+            if (cnt) atomic_add_agent(super + e, cnt);
+        }
+    }
     __syncthreads();
 }
 

@@ -106,8 +106,13 @@ static_assert(kSchedMembers + 2 * kXcds * kSchedLine <= kSchedReady, "member wor
 // ticks of the 100 MHz wall clock a waiter records an error and proceeds.
 constexpr unsigned long long kWaitTicks = 300000000ull;   // 3 s
 // LDS header of the expert phase (bytes)
-constexpr size_t kLdsMt = 1536, kLdsQueue = 256, kLdsSeg = 8 * (2 * 16 * kMaxGateGroups);
-constexpr size_t kFusedLdsHeader = kLdsMt + kLdsQueue + kLdsSeg;
+// rows kept per expert u32[Ep] | row blocks u16[Ep] | queue words (kLdsQueue bytes) | segments [2 Ep],
+// with Ep = the expert count rounded up to 64, at least 256
+constexpr size_t kLdsQueue = 256;
+constexpr uint32_t kMaxExperts = 512;   // the header and the tiles of the narrow variant share 160 KB of LDS
+__host__ __device__ inline uint32_t lds_experts(uint32_t E) { return E <= 256 ? 256u : (E + 63) / 64 * 64; }
+__host__ __device__ inline size_t lds_queue_offset(uint32_t E) { return size_t(6) * lds_experts(E); }
+__host__ __device__ inline size_t fused_lds_header(uint32_t E) { return lds_queue_offset(E) + kLdsQueue + size_t(16) * lds_experts(E); }
 
 struct Segment {
     uint16_t expert;
@@ -427,7 +432,8 @@ __device__ __forceinline__ void expert_loop(const LayerParams& p, char* smem, ui
 template <typename T, int NG>
 __global__ __launch_bounds__(TileShape<T>::kThreads) void gate_kernel(const LayerParams p) {
     extern __shared__ __attribute__((aligned(16))) float gate_smem[];
-    gate_unit<T, NG, TileShape<T>::kThreads / kWave>(p, blockIdx.x, gate_smem);
+    if constexpr (NG == 0) gate_unit_wide<T, TileShape<T>::kThreads / kWave>(p, blockIdx.x, gate_smem);
+    else gate_unit<T, NG, TileShape<T>::kThreads / kWave>(p, blockIdx.x, gate_smem);
 }
 
 __global__ __launch_bounds__(kPhaseThreads) void slot_kernel(const LayerParams p) {
@@ -523,7 +529,8 @@ __global__ __launch_bounds__((TileShape<T, V>::kThreads), (TileShape<T, V>::kPer
         for (uint32_t i = tid; i < p.E * mt_max; i += kThreads) sched[kSchedReady + i] = 0u;
     }
     for (uint32_t unit = blockIdx.x; unit < ceil_div_u32(p.n_gate_tiles, gate_unit_blocks<NG>()); unit += nwg)
-        gate_unit<T, NG, int(kWaves)>(p, unit, reinterpret_cast<float*>(smem));
+        if constexpr (NG == 0) gate_unit_wide<T, int(kWaves)>(p, unit, reinterpret_cast<float*>(smem));
+        else gate_unit<T, NG, int(kWaves)>(p, unit, reinterpret_cast<float*>(smem));
     if (tid == 0) stamp[1] = wall_clock64();
     grid_barrier(sched, 0, seq, nwg);
     if (tid == 0) stamp[2] = wall_clock64();
@@ -541,9 +548,9 @@ __global__ __launch_bounds__((TileShape<T, V>::kThreads), (TileShape<T, V>::kPer
 
     // ---- phase 2: expert tiles from the per-XCD queues (by ticket, or by stride in the static schedule)
     // LDS map: row blocks per expert | queue starts, totals, task | segments | GEMM tile
-    uint32_t* s_rows = reinterpret_cast<uint32_t*>(smem);                       // [E], E <= 256: rows kept
-    uint16_t* s_mt = reinterpret_cast<uint16_t*>(smem + 1024);                  // [E] row blocks
-    uint32_t* s_qseg = reinterpret_cast<uint32_t*>(smem + kLdsMt);              // [9] first segment of each queue
+    uint32_t* s_rows = reinterpret_cast<uint32_t*>(smem);                       // [E] rows kept
+    uint16_t* s_mt = reinterpret_cast<uint16_t*>(smem + 4 * lds_experts(p.E));  // [E] row blocks
+    uint32_t* s_qseg = reinterpret_cast<uint32_t*>(smem + lds_queue_offset(p.E));   // [9] first segment of each queue
     uint32_t* s_qtot = s_qseg + 16;                                             // [8] tickets in each queue
     uint32_t* s_task = s_qtot + 8;                                              // [kTaskWords] task broadcast slot
     uint32_t* s_qup = s_task + kTaskWords;                                      // [8] up-projection tickets in each queue
@@ -553,8 +560,8 @@ __global__ __launch_bounds__((TileShape<T, V>::kThreads), (TileShape<T, V>::kPer
     // stay occupied through the GEMM main loop.
     uint32_t* s_static = s_qup + 8;
     static_assert((16 + 8 + kTaskWords + 8 + 6) * 4 <= kLdsQueue, "queue header");
-    Segment* s_seg = reinterpret_cast<Segment*>(smem + kLdsMt + kLdsQueue);     // at most 2*E segments
-    char* s_gemm = smem + kFusedLdsHeader;
+    Segment* s_seg = reinterpret_cast<Segment*>(smem + lds_queue_offset(p.E) + kLdsQueue);   // at most 2*E segments
+    char* s_gemm = smem + fused_lds_header(p.E);
     const uint32_t tn_up = ceil_div_u32(p.I, BN), tn_down = ceil_div_u32(p.H, BN);
 
     // The queues of the expert phase are set up while this workgroup waits for the others to finish
@@ -716,7 +723,7 @@ __global__ __launch_bounds__((TileShape<T, V>::kThreads), (TileShape<T, V>::kPer
 
 template <typename T, int NG, int V>
 size_t fused_smem_bytes(uint32_t E) {
-    size_t need = kFusedLdsHeader + gemm_smem_bytes<T, V>();
+    size_t need = fused_lds_header(E) + gemm_smem_bytes<T, V>();
     const size_t gate = gate_smem_floats<NG>(TileShape<T>::kThreads / kWave) * sizeof(float);
     const size_t slots = (TileShape<T>::kThreads / kWave) * size_t(E) * sizeof(uint32_t);
     if (gate > need) need = gate;
@@ -755,8 +762,10 @@ hipError_t dispatch_variant(const LayerParams& p, F&& f) {
     return f(std::integral_constant<int, 0>{});
 }
 
+// Calls f(integral_constant<int, NG>) with the expert groups of the gate: 0 = the wide gate.
 template <typename F>
 hipError_t dispatch_groups(uint32_t E, F&& f) {
+    if (E > 16 * kMaxGateGroups) return f(std::integral_constant<int, 0>{});
     switch (gate_groups(E)) {
         case 1: return f(std::integral_constant<int, 1>{});
         case 2: return f(std::integral_constant<int, 2>{});
@@ -769,8 +778,9 @@ hipError_t dispatch_groups(uint32_t E, F&& f) {
 }  // namespace
 
 const char* unsupported_reason(uint32_t E, uint32_t k) {
-    (void)k;
-    if (E > 16 * kMaxGateGroups) return "num_experts > 256 is not supported by the gate kernel of this build";
+    if (E > kMaxExperts) return "num_experts > 512 is not supported by this build (LDS tables of the persistent kernel)";
+    if (E > 16 * kMaxGateGroups && k > kWideGateMaxK)
+        return "expert_top_k > 32 with num_experts > 256 is not supported by the gate kernel of this build";
     return nullptr;
 }
 

@@ -7,7 +7,7 @@ namespace kleos_amd {
 
 constexpr int kGateTileTokens = 16;   // tokens per gate tile (one MFMA column block)
 constexpr int kSuperTiles = 32;       // gate tiles per coarse count row (512 tokens)
-constexpr int kMaxGateGroups = 16;    // 16 experts per group -> gate handles E <= 256
+constexpr int kMaxGateGroups = 16;    // 16 experts per group: up to 256 experts keep their logits in registers
 
 // Work item of the expert phase: one output tile of the up- or down-projection.
 struct TileTask {

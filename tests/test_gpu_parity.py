@@ -151,6 +151,9 @@ CASES = [
     (256, 192, 320, 12, 3, 1.0, 1, 1, 3, 0.1),     # fp16, gelu + biases, ragged sizes
     (512, 256, 256, 64, 2, 1.0, 1, 0, 3, 0.0),     # fp16, E = 64, several K slices
     (2048, 192, 320, 2, 2, 1.0, 1, 1, 2, 0.1),     # 2048 rows per expert: the tile variant of large experts
+    (512, 128, 64, 320, 8, 1.0, 1, 0, 2, 0.0),     # E > 256: the gate in passes of 256 experts
+    (256, 192, 64, 512, 6, 2.0, 1, 1, 2, 0.1),     # E = 512, cf = 2, gelu + biases
+    (256, 64, 64, 384, 4, 1.0, 1, 0, 0, 0.0),      # fp32, E = 384
 ]
 
 
@@ -411,7 +414,7 @@ def test_fine_e256_top8_full_size(mode):
 
 
 # ------------------------------------------------------------------ training mode
-@pytest.mark.parametrize("E,k,S", [(16, 2, 1024), (64, 2, 2048), (130, 8, 512)])
+@pytest.mark.parametrize("E,k,S", [(16, 2, 1024), (64, 2, 2048), (130, 8, 512), (384, 4, 512)])
 def test_training_mode_gate_loss(E, k, S):
     """is_training: 1 adds the load-balancing loss of the gate (gate.cuh:608-635, 700-705, 763-773):
     checked against the oracle evaluated on the GPU's own logits, identical in both modes (every
