@@ -318,16 +318,34 @@ __device__ __forceinline__ void gate_unit_wide(const LayerParams& p, uint32_t un
         f32x4 acc[NG];
 #pragma unroll
         for (int g = 0; g < NG; ++g) acc[g] = f32x4{0.f, 0.f, 0.f, 0.f};
-        for (uint32_t s = s0; s < s1; ++s) {
+        // weight rows past the padded expert count re-read its last row; their logits are never stored
+        auto wrow = [&](int g) {
+            const uint32_t r = e0 + 16 * g + col;
+            return static_cast<const T*>(p.wg) + size_t(r < p.PX ? r : p.PX - 1) * H + chunk * kPer;
+        };
+        // the loads of U steps are issued together before their matrix instructions
+        constexpr int U = 2;
+        uint32_t s = s0;
+        for (; s + U <= s1; s += U) {
+            u32x4 xb[U], wa[U][NG];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const uint32_t off = (s + u) * kStepK;
+                xb[u] = load16(xrow + off);
+#pragma unroll
+                for (int g = 0; g < NG; ++g) wa[u][g] = load16(wrow(g) + off);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+#pragma unroll
+                for (int g = 0; g < NG; ++g) acc[g] = mma16_step(wa[u][g], xb[u], acc[g], T{});
+        }
+        for (; s < s1; ++s) {
             const uint32_t off = s * kStepK;
             const u32x4 xb = load16(xrow + off);
 #pragma unroll
-            for (int g = 0; g < NG; ++g) {
-                // weight rows past the padded expert count re-read its last row; their logits are never stored
-                const uint32_t r = e0 + 16 * g + col;
-                const T* wrow = static_cast<const T*>(p.wg) + size_t(r < p.PX ? r : p.PX - 1) * H + chunk * kPer;
-                acc[g] = mma16_step(load16(wrow + off), xb, acc[g], T{});
-            }
+            for (int g = 0; g < NG; ++g) acc[g] = mma16_step(load16(wrow(g) + off), xb, acc[g], T{});
         }
         float* dst = smem + part * (NG * 4 * kWave);
 #pragma unroll
