@@ -93,7 +93,9 @@ int kleos_config_derive(kleos_config_t* cfg);
 /* Replaces kleos::initialize() (csrc/include/kleos/bootstrap.cuh:533-547): validates the config,
  * selects the device, creates the library stream and allocates every scratch arena (routing
  * tables, intermediate activations, scheduler counters) the forward needs, as the reference's
- * Bookkeeping arenas are (bootstrap.cuh:377-391). Fails with KLEOS_ESTATE "Already Initialized". */
+ * Bookkeeping arenas are (bootstrap.cuh:377-391). Fails with KLEOS_ESTATE "Already Initialized",
+ * and with KLEOS_EUNSUPPORTED for what this build leaves out: tf32, more than 512 experts, top-k
+ * above 32 together with more than 256 experts. */
 int kleos_initialize(const char* config_json_path);
 int kleos_initialize_cfg(const kleos_config_t* cfg);
 /* Replaces kleos::finalize() (bootstrap.cuh:562-588): drains the stream, frees every arena. */
