@@ -453,6 +453,14 @@ def test_training_mode_gate_loss(E, k, S):
         np.testing.assert_array_equal(outp, out)
 
 
+def test_configurations_this_build_leaves_out_are_refused():
+    for keys in (_keys(256, 128, 64, 576, 2), _keys(256, 128, 64, 320, 40)):
+        with pytest.raises(ka.KleosError) as ei:
+            ka.initialize(keys)
+        assert ei.value.code == ka._capi.KLEOS_EUNSUPPORTED
+        assert not ka.is_initialized()
+
+
 def test_gate_loss_needs_training_mode():
     keys = _keys(256, 128, 128, 8, 2)
     d = ka.initialize(keys)
