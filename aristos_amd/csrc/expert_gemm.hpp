@@ -143,7 +143,10 @@ __device__ __forceinline__ void epilogue16(const TileOut& t, f32x16 (&acc)[WN / 
 }
 
 // ISSUE: over how many K steps of a slice the loads of the slice STAGES-1 ahead are issued.
-template <typename E, int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES, int ISSUE>
+// STREAM_B: the weight rows are loaded with the non-temporal cache policy: read once (or by a
+// neighbour at the same moment), they pass through the L2 without displacing the activation rows
+// that are shared (7.0 against 6.4 TB/s on a read-only stream of this shape).
+template <typename E, int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES, int ISSUE, bool STREAM_B>
 struct Gemm16 {
     typedef typename Elem16<E>::vec8 vec8;
     typedef typename Elem16<E>::vec4 vec4;
@@ -161,6 +164,7 @@ struct Gemm16 {
     static constexpr int kSmemBytes = STAGES * kStage + 2 * kBiasBytes;
     static constexpr int LA = BM / (kRowsPerLoad * kWaves), LB = BN / (kRowsPerLoad * kWaves);
     static constexpr int kLoadsPerSlice = LA + LB;                 // per wavefront
+    static constexpr int kNonTemporal = 2;                         // cache policy bit nt of a load
     static constexpr int kSliceK = BK;                             // values of K per slice
     static constexpr int kSteps = BK / 16;                         // matrix instructions consume 16 values of K
     static constexpr int kPanelRows = kEpiloguePanelRows;          // epilogue staging: 32 rows x 64 columns per wavefront
@@ -208,7 +212,8 @@ struct Gemm16 {
 #pragma unroll
         for (int i = 0; i < LB; ++i)
             if (i * parts / LB == part)
-                __builtin_amdgcn_global_load_lds((global_cptr)(t.pb[i] + k0), (lds_ptr)(sb + 1024 * (wave + kWaves * i)), 16, 0, 0);
+                __builtin_amdgcn_global_load_lds((global_cptr)(t.pb[i] + k0), (lds_ptr)(sb + 1024 * (wave + kWaves * i)), 16, 0,
+                                                 STREAM_B ? kNonTemporal : 0);
     }
 
     // Per-lane source addresses, the load of the bias into LDS slot `bias_slot`, then the loads of

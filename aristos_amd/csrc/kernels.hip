@@ -44,9 +44,12 @@ constexpr int kXcds = 8;
 // variant 0 with all loads of the next slice issued at the first K step (measured on the 8-expert
 // top-2 shape with hidden size 4096: 3.8 ms against 3.9 ms with two issue steps and 4.0 with four;
 // at the headline shape, whose weights stream from HBM, one step loses 6 % against two).
+// Variants 0 and 1 load their weight rows non-temporally (headline 378 against 390 us per forward,
+// the 16-expert shape 192 against 196, the 256-expert shape 3.43 against 3.48 ms); variant 2, whose
+// weight tiles are shared by eight workgroups and more, does not (4.06 against 4.01 ms with it).
 template <typename E, int V>
-using GemmCfg = std::conditional_t<V == 0, Gemm16<E, 256, 256, 2, 4, 64, 2, 2>,
-                std::conditional_t<V == 1, Gemm16<E, 128, 256, 2, 4, 64, 3, 1>, Gemm16<E, 256, 256, 2, 4, 64, 2, 1>>>;
+using GemmCfg = std::conditional_t<V == 0, Gemm16<E, 256, 256, 2, 4, 64, 2, 2, true>,
+                std::conditional_t<V == 1, Gemm16<E, 128, 256, 2, 4, 64, 3, 1, true>, Gemm16<E, 256, 256, 2, 4, 64, 2, 1, false>>>;
 constexpr int kBN = 256;
 constexpr int kGemmThreads = GemmCfg<bf16_t, 0>::kThreads;
 static_assert(GemmCfg<bf16_t, 1>::kThreads == kGemmThreads && GemmCfg<bf16_t, 2>::kThreads == kGemmThreads,
