@@ -50,3 +50,13 @@ def test_initialize_without_a_gpu_raises():
         ka.initialize(ka.KleosConfig(sequence_len=128, hidden_size=64, intermediate_size=64, num_experts=4))
     assert ei.value.code == _capi.KLEOS_EHIP
     assert not ka.is_initialized()
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU's share only: asked for more, it says so and exits (no GPU needed)."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    proc = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert proc.returncode == 2
+    assert "single-GPU" in proc.stderr and proc.stdout.strip() == ""
