@@ -65,6 +65,10 @@ SYMBOLS = {
     "kleos_debug_copy_to_host": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t]),
     "kleos_scheduler_stats": (C.c_int, [C.POINTER(C.c_double)]),
     "kleos_measure_throughput": (C.c_int, [C.c_uint32, C.POINTER(C.c_float), C.POINTER(C.c_float)]),
+    "kleos_measure_throughput_output": (C.c_int, [C.c_uint32, C.POINTER(C.c_float), C.POINTER(C.c_float), C.c_void_p,
+                                                  C.c_size_t]),
+    "kleos_debug_set_wait_ticks": (C.c_int, [C.c_ulonglong]),
+    "kleos_debug_skip_launch_number": (C.c_int, []),
     "kleos_gate_loss": (C.c_int, [C.POINTER(C.c_float), C.POINTER(C.c_float), C.POINTER(C.c_float)]),
     "kleos_phase_stamps": (C.c_int, [C.POINTER(C.c_ulonglong), C.c_uint32, C.POINTER(C.c_uint32)]),
     "kleos_phase_times": (C.c_int, [C.POINTER(C.c_float)]),

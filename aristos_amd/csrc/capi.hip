@@ -29,6 +29,7 @@ struct Context {
     uint32_t fused_seq = 0;         // fused forwards issued (grid-barrier arrival base)
     int mode = KLEOS_MODE_FUSED;
     int schedule = KLEOS_SCHEDULE_AUTO;
+    size_t zero_begin = 0, zero_end = 0;   // the part of the arena that holds counters (starts as zeros)
     float phase_ms[5] = {0, 0, 0, 0, 0};
     double sched_stats[6] = {0, 0, 0, 0, 0, 0};
 };
@@ -44,6 +45,7 @@ Context* g_ctx = nullptr;   // one context per process, like the reference's glo
     } while (0)
 
 constexpr uint32_t kMaxWorkgroups = 1024;   // persistent grid never exceeds CUs x 2
+constexpr unsigned long long kDefaultWaitTicks = 300000000ull;   // 3 s of the 100 MHz wall clock
 
 size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
@@ -82,14 +84,20 @@ ArenaLayout layout_arena(const kleos_config_t& c, uint32_t n_tiles, uint32_t n_s
 }
 
 // After a synchronisation: did a persistent kernel give up waiting on its scheduler counters?
+// A launch that gave up leaves the monotonic barrier counters, the member counts and the count of
+// static launches short of what the launch numbers imply, so every counter goes back to zero and
+// the launch numbers with them: the next forward starts from the state of a fresh context.
 int check_scheduler(Context& c) {
     uint32_t flag = 0;
     hipError_t e = hipMemcpy(&flag, c.base.sched + sched_error_word(), 4, hipMemcpyDeviceToHost);
     if (e != hipSuccess) return fail(KLEOS_EHIP, "scheduler check: %s", hipGetErrorString(e));
     if (flag) {
-        (void)hipMemset(c.base.sched + sched_error_word(), 0, 4);
+        e = hipMemset(c.arena + c.zero_begin, 0, c.zero_end - c.zero_begin);
+        c.launch_seq = 0;
+        c.fused_seq = 0;
+        if (e != hipSuccess) return fail(KLEOS_EHIP, "scheduler reset: %s", hipGetErrorString(e));
         return fail(KLEOS_EHIP, "persistent kernel: a bounded wait on the tile scheduler expired; "
-                                "the outputs of that launch are invalid");
+                                "the outputs of that launch are invalid (scheduler state reset)");
     }
     return KLEOS_OK;
 }
@@ -189,6 +197,9 @@ extern "C" int kleos_initialize_cfg(const kleos_config_t* user_cfg) {
     const ArenaLayout L = layout_arena(cfg, p.n_gate_tiles, p.n_super);
     KLEOS_HIP_BAIL(hipMalloc(reinterpret_cast<void**>(&c->arena), L.total));
     c->arena_bytes = L.total;
+    c->zero_begin = L.zero_begin;
+    c->zero_end = L.zero_end;
+    p.wait_ticks = kDefaultWaitTicks;
     KLEOS_HIP_BAIL(hipMemsetAsync(c->arena + L.zero_begin, 0, L.zero_end - L.zero_begin, c->stream));
     KLEOS_HIP_BAIL(hipStreamSynchronize(c->stream));
     char* a = c->arena;
@@ -397,10 +408,19 @@ extern "C" int kleos_scheduler_stats(double stats[6]) {
 }
 
 extern "C" int kleos_measure_throughput(uint32_t trials, float* median_ms, float* throughput) {
+    return kleos_measure_throughput_output(trials, median_ms, throughput, nullptr, 0);
+}
+
+extern "C" int kleos_measure_throughput_output(uint32_t trials, float* median_ms, float* throughput, void* y_host,
+                                               size_t y_bytes) {
     if (int rc = require_ctx("kleos_measure_throughput")) return rc;
     if (!median_ms || !throughput || trials == 0 || trials > 1024)
         return fail(KLEOS_EINVAL, "kleos_measure_throughput: need result pointers and 1 <= trials <= 1024");
     Context& c = *g_ctx;
+    if (y_bytes && !y_host) return fail(KLEOS_EINVAL, "kleos_measure_throughput_output: null result buffer");
+    if (y_bytes > size_t(c.cfg.pEC) * c.cfg.H * c.cfg.elem_bytes)
+        return fail(KLEOS_EINVAL, "kleos_measure_throughput_output: the probe's result holds %zu bytes",
+                    size_t(c.cfg.pEC) * c.cfg.H * c.cfg.elem_bytes);
     KLEOS_HIP(hipSetDevice(c.device));
     // One expert at full padded capacity, as the reference's probe (throughput.cuh:104-170):
     // M = pEC rows, up-projection to I columns over K = H, activation, down-projection back to H.
@@ -447,6 +467,7 @@ extern "C" int kleos_measure_throughput(uint32_t trials, float* median_ms, float
         std::sort(ms.begin(), ms.end());
         *median_ms = ms[trials / 2];                          // throughput.cuh:166 (findMedian)
         *throughput = *median_ms > 0.f ? 1.0f / *median_ms : 0.f;
+        if (y_bytes) KLEOS_HIP(hipMemcpy(y_host, buf + o_y, y_bytes, hipMemcpyDeviceToHost));
         return KLEOS_OK;
     };
     rc = body();
@@ -454,6 +475,18 @@ extern "C" int kleos_measure_throughput(uint32_t trials, float* median_ms, float
     for (auto& e : ev) if (e) (void)hipEventDestroy(e);
     (void)hipFree(buf);
     return rc;
+}
+
+extern "C" int kleos_debug_set_wait_ticks(unsigned long long ticks) {
+    if (int rc = require_ctx("kleos_debug_set_wait_ticks")) return rc;
+    g_ctx->base.wait_ticks = ticks ? ticks : kDefaultWaitTicks;
+    return KLEOS_OK;
+}
+
+extern "C" int kleos_debug_skip_launch_number(void) {
+    if (int rc = require_ctx("kleos_debug_skip_launch_number")) return rc;
+    g_ctx->fused_seq++;
+    return KLEOS_OK;
 }
 
 extern "C" int kleos_gate_loss(float* loss, float* mean_prob, float* mean_count) {

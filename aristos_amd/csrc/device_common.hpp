@@ -87,16 +87,19 @@ __device__ __forceinline__ f32x4 mma16_step(u32x4 a, u32x4 b, f32x4 acc, float) 
     return acc;
 }
 
+// Waits until at most N of this wavefront's vector-memory operations (loads and stores alike) are
+// outstanding.
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+    static_assert(N >= 0 && N < 64);
+    // s_waitcnt simm16: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] at [15:14]
+    __builtin_amdgcn_s_waitcnt(0x0f70 | (N & 15) | ((N >> 4) << 14));
+}
+
 // Device-scope (agent) atomics: the scheduler counters are shared by workgroups on different
 // XCDs, whose L2 caches are not coherent with each other for ordinary loads and stores.
 __device__ __forceinline__ uint32_t atomic_add_agent(uint32_t* p, uint32_t v) {
     return __hip_atomic_fetch_add(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ uint32_t atomic_add_release(uint32_t* p, uint32_t v) {
-    return __hip_atomic_fetch_add(p, v, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ uint32_t atomic_load_acquire(const uint32_t* p) {
-    return __hip_atomic_load(p, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
 }
 __device__ __forceinline__ uint32_t atomic_load_relaxed(const uint32_t* p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

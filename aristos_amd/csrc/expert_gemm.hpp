@@ -42,14 +42,6 @@ namespace kleos_amd {
 typedef const __attribute__((address_space(1))) void* global_cptr;
 typedef __attribute__((address_space(3))) void* lds_ptr;
 
-// Waits until at most N of this wavefront's vector-memory operations are outstanding.
-template <int N>
-__device__ __forceinline__ void wait_vmcnt() {
-    static_assert(N >= 0 && N < 64);
-    // s_waitcnt simm16: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt[5:4] at [15:14]
-    __builtin_amdgcn_s_waitcnt(0x0f70 | (N & 15) | ((N >> 4) << 14));
-}
-
 // A 16-bit Element seen only as storage: addresses are computed in units of it, values are
 // interpreted by the Element type the tile is instantiated with.
 typedef uint16_t elem16_t;

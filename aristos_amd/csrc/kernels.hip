@@ -105,9 +105,9 @@ constexpr uint32_t kScheduleAuto = 0, kScheduleStatic = 2;   // anything else: d
 static_assert(kSchedBar + kGridBarriers * kSchedLine <= kSchedTicket, "barrier words");
 static_assert(kSchedGroup + kGridBarriers * kXcds * kSchedLine <= kSchedMembers, "barrier group words");
 static_assert(kSchedMembers + 2 * kXcds * kSchedLine <= kSchedReady, "member words");
-// Every wait in the persistent kernel is bounded so that the grid always drains: after this many
-// ticks of the 100 MHz wall clock a waiter records an error and proceeds.
-constexpr unsigned long long kWaitTicks = 300000000ull;   // 3 s
+// Every wait in the persistent kernel is bounded so that the grid always drains: after
+// LayerParams::wait_ticks ticks of the 100 MHz wall clock (3 s unless the host says otherwise) a
+// waiter records an error and proceeds.
 // LDS header of the expert phase (bytes)
 // rows kept per expert u32[Ep] | row blocks u16[Ep] | queue words (kLdsQueue bytes) | segments [2 Ep],
 // with Ep = the expert count rounded up to 64, at least 256
@@ -124,14 +124,14 @@ struct Segment {
     uint32_t start;     // first ticket of the segment inside its queue
 };
 
-// Spins (thread 0 only) until pred() holds or the wait bound expires.
+// Spins (one thread) until pred() holds or `ticks` ticks of the wall clock have passed.
 template <typename Pred>
-__device__ __forceinline__ void bounded_wait(uint32_t* sched, Pred&& pred) {
+__device__ __forceinline__ void bounded_wait(uint32_t* sched, unsigned long long ticks, Pred&& pred) {
     if (pred()) return;
     const unsigned long long t0 = wall_clock64();
     while (!pred()) {
         __builtin_amdgcn_s_sleep(2);
-        if (wall_clock64() - t0 > kWaitTicks) {
+        if (wall_clock64() - t0 > ticks) {
             atomic_store_relaxed(sched + kSchedError, 1u);
             return;
         }
@@ -149,8 +149,12 @@ __device__ __forceinline__ void bounded_wait(uint32_t* sched, Pred&& pred) {
 // wait. The arrival and the wait are the business of the first lane of the last wavefront, so that
 // the wavefronts `between` keeps busy (it may hold workgroup barriers) do not sit behind the
 // arrival's trips to memory longer than they must.
+// Every wavefront first waits for its own outstanding stores: the workgroup barrier does not, and
+// the leader's release covers only what has left the other wavefronts' queues by then.
 template <typename Between>
-__device__ __forceinline__ void grid_barrier(uint32_t* sched, uint32_t which, uint32_t seq, uint32_t nwg, Between&& between) {
+__device__ __forceinline__ void grid_barrier(uint32_t* sched, unsigned long long ticks, uint32_t which, uint32_t seq, uint32_t nwg,
+                                             Between&& between) {
+    wait_vmcnt<0>();
     __syncthreads();
     const bool leader = threadIdx.x == blockDim.x - kWave;
     if (leader) {
@@ -169,7 +173,7 @@ __device__ __forceinline__ void grid_barrier(uint32_t* sched, uint32_t which, ui
         const uint32_t groups = nwg < uint32_t(kXcds) ? nwg : uint32_t(kXcds);
         uint32_t* all = sched + kSchedBar + which * kSchedLine;
         const uint32_t target = (seq + 1u) * groups;
-        bounded_wait(sched, [&] { return int32_t(atomic_load_relaxed(all) - target) >= 0; });
+        bounded_wait(sched, ticks, [&] { return int32_t(atomic_load_relaxed(all) - target) >= 0; });
     }
     __syncthreads();
     // No device-scope acquire here: it would invalidate the whole L2 of the XCD (tens of
@@ -178,8 +182,8 @@ __device__ __forceinline__ void grid_barrier(uint32_t* sched, uint32_t which, ui
     asm volatile("buffer_inv sc0" ::: "memory");
 }
 
-__device__ __forceinline__ void grid_barrier(uint32_t* sched, uint32_t which, uint32_t seq, uint32_t nwg) {
-    grid_barrier(sched, which, seq, nwg, [] {});
+__device__ __forceinline__ void grid_barrier(uint32_t* sched, unsigned long long ticks, uint32_t which, uint32_t seq, uint32_t nwg) {
+    grid_barrier(sched, ticks, which, seq, nwg, [] {});
 }
 
 // Tokens the gate routed to expert e in this launch, dropped ones included: the sum of the coarse
@@ -202,14 +206,15 @@ __device__ __forceinline__ uint32_t routed_count(const LayerParams& p, uint32_t 
 // Barrier among the `members` workgroups that run on XCD `xcd`, the `runs`-th time it is held on this
 // arena (counted from 0). The static schedule holds it between the two projections: a down tile
 // reads h1 rows that only workgroups of its own XCD stored.
-__device__ __forceinline__ void xcd_barrier(uint32_t* sched, uint32_t xcd, uint32_t runs, uint32_t members) {
+__device__ __forceinline__ void xcd_barrier(uint32_t* sched, unsigned long long ticks, uint32_t xcd, uint32_t runs, uint32_t members) {
+    wait_vmcnt<0>();   // the h1 stores of every wavefront, before the leader's release
     __syncthreads();
     if (threadIdx.x == 0) {
         uint32_t* arrived = sched + kSchedGroup + ((kGridBarriers - 1) * kXcds + xcd) * kSchedLine;
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
         atomic_add_agent(arrived, 1u);
         const uint32_t target = (runs + 1u) * members;
-        bounded_wait(sched, [&] { return int32_t(atomic_load_relaxed(arrived) - target) >= 0; });
+        bounded_wait(sched, ticks, [&] { return int32_t(atomic_load_relaxed(arrived) - target) >= 0; });
     }
     __syncthreads();
     asm volatile("buffer_inv sc0" ::: "memory");   // drop this CU's L1; the rows are current in the XCD's L2
@@ -294,6 +299,7 @@ __device__ __forceinline__ uint32_t first_k_slice(uint32_t e, uint32_t E, uint32
 struct Readiness {
     uint32_t* sched;      // nullptr: no cross-tile dependencies inside this launch (phased mode)
     uint32_t mt_max, tn_up;
+    unsigned long long ticks;   // bound of a wait for a row block
     __device__ __forceinline__ uint32_t* counter(const Task& t) const { return sched + kSchedReady + t.e * mt_max + t.mtile; }
     // A counter holds the stored tiles of the row block in its low half and, in its high half, how
     // many of them were stored by a workgroup on a foreign XCD (from whose L2 they were written back
@@ -328,7 +334,7 @@ __device__ __forceinline__ void expert_loop(const LayerParams& p, char* smem, ui
         const unsigned long long t0 = wall_clock64();
         if (tid == 0) {
             uint32_t seen = t.dep;
-            bounded_wait(rd.sched, [&] { seen = atomic_load_relaxed(rd.counter(t)); return rd.complete(seen); });
+            bounded_wait(rd.sched, rd.ticks, [&] { seen = atomic_load_relaxed(rd.counter(t)); return rd.complete(seen); });
             s_task[kTaskWords - 1] = seen;
         }
         __syncthreads();
@@ -421,6 +427,7 @@ __device__ __forceinline__ void expert_loop(const LayerParams& p, char* smem, ui
             if (o.act == 0) gemm_tile_f32<0>(o.a, o.idx, p.S, o.lda, o.m_valid, o.w, o.K, o.n_valid, o.bias, o.c, o.ldc, o.K, smem);
             else if (o.act == 1) gemm_tile_f32<1>(o.a, o.idx, p.S, o.lda, o.m_valid, o.w, o.K, o.n_valid, o.bias, o.c, o.ldc, o.K, smem);
             else gemm_tile_f32<2>(o.a, o.idx, p.S, o.lda, o.m_valid, o.w, o.K, o.n_valid, o.bias, o.c, o.ldc, o.K, smem);
+            wait_vmcnt<0>();   // the tile's stores, in every wavefront, before it is counted
             __syncthreads();
             publish(t);
         }
@@ -485,7 +492,7 @@ __global__ __launch_bounds__((TileShape<T, V>::kThreads), (TileShape<T, V>::kPer
         }
         return broadcast_task(s_task, t);
     };
-    expert_loop<T, V>(p, gemm_smem + kPhasedGemmHeader, s_task, Readiness{nullptr, 0, 0}, nullptr, next, [] {});
+    expert_loop<T, V>(p, gemm_smem + kPhasedGemmHeader, s_task, Readiness{nullptr, 0, 0, 0}, nullptr, next, [] {});
 }
 
 template <typename T>
@@ -535,7 +542,7 @@ __global__ __launch_bounds__((TileShape<T, V>::kThreads), (TileShape<T, V>::kPer
         if constexpr (NG == 0) gate_unit_wide<T, int(kWaves)>(p, unit, reinterpret_cast<float*>(smem));
         else gate_unit<T, NG, int(kWaves)>(p, unit, reinterpret_cast<float*>(smem));
     if (tid == 0) stamp[1] = wall_clock64();
-    grid_barrier(sched, 0, seq, nwg);
+    grid_barrier(sched, p.wait_ticks, 0, seq, nwg);
     if (tid == 0) stamp[2] = wall_clock64();
 
     // ---- phase 1: slots in token order
@@ -572,7 +579,7 @@ __global__ __launch_bounds__((TileShape<T, V>::kThreads), (TileShape<T, V>::kPer
     // per XCD) has been complete since the first barrier.
     const uint32_t members = nwg / kXcds;
     bool use_static = false;
-    grid_barrier(sched, 1, seq, nwg, [&] {
+    grid_barrier(sched, p.wait_ticks, 1, seq, nwg, [&] {
         // how many workgroups every XCD holds: asked for first, so that the answers travel together
         // with the routed counts below
         uint32_t seen[kXcds] = {};
@@ -659,7 +666,7 @@ __global__ __launch_bounds__((TileShape<T, V>::kThreads), (TileShape<T, V>::kPer
     uint32_t q_off = 0;   // queues already found empty, starting from this workgroup's own XCD
     uint32_t q_dead = 0;  // bit q: queue q was seen exhausted
     bool q_scanned = false;
-    const Readiness rd{use_static ? nullptr : sched, mt_max, tn_up};
+    const Readiness rd{use_static ? nullptr : sched, mt_max, tn_up, p.wait_ticks};
     auto decode = [&](Task& t, uint32_t q, uint32_t ticket) {
         uint32_t sg = s_qseg[q];
         const uint32_t sg_end = s_qseg[q + 1];
@@ -710,9 +717,9 @@ __global__ __launch_bounds__((TileShape<T, V>::kThreads), (TileShape<T, V>::kPer
         }
         return broadcast_task(s_task, t);
     };
-    expert_loop<T, V>(p, s_gemm, s_task, rd, stamp + 8, next, [&] { xcd_barrier(sched, xcd, s_static[2], members); });
+    expert_loop<T, V>(p, s_gemm, s_task, rd, stamp + 8, next, [&] { xcd_barrier(sched, p.wait_ticks, xcd, s_static[2], members); });
     if (tid == 0) stamp[5] = wall_clock64();
-    grid_barrier(sched, 2, seq, nwg);
+    grid_barrier(sched, p.wait_ticks, 2, seq, nwg);
     if (tid == 0) stamp[6] = wall_clock64();
     // every workgroup read the count when it started, before the first barrier
     if (use_static && blockIdx.x == 0 && tid == 0) atomic_store_relaxed(sched + kSchedStaticRuns, s_static[2] + 1u);

@@ -9,14 +9,6 @@ constexpr int kGateTileTokens = 16;   // tokens per gate tile (one MFMA column b
 constexpr int kSuperTiles = 32;       // gate tiles per coarse count row (512 tokens)
 constexpr int kMaxGateGroups = 16;    // 16 experts per group: up to 256 experts keep their logits in registers
 
-// Work item of the expert phase: one output tile of the up- or down-projection.
-struct TileTask {
-    uint16_t expert;
-    uint16_t kind;      // 0 up-projection, 1 down-projection
-    uint32_t row0;      // first slot (row inside the expert's buffer)
-    uint32_t col0;      // first output column
-};
-
 struct LayerParams {
     // ---- configuration (derived as the reference's struct ACC, types.cuh:471-507)
     uint32_t S, H, I, E, k, PX, EC, cap_rows, act;
@@ -53,6 +45,7 @@ struct LayerParams {
     uint32_t* sched;          // counters, see the scheduler section of kernels.hip
     unsigned long long* stamps;   // [workgroups][8] 100 MHz wall-clock stamps of the phase boundaries
     uint32_t epoch;           // launch parity, selects the live half of double-buffered counters
+    unsigned long long wait_ticks;   // bound of every in-kernel wait, in ticks of the 100 MHz wall clock
 };
 
 }  // namespace kleos_amd

@@ -50,6 +50,27 @@ uint16_t to_bf16(float v) {
     return uint16_t(u >> 16);
 }
 
+// fp32 -> IEEE binary16 bits, round to nearest even; overflow to infinity, gradual underflow.
+uint16_t to_f16(float v) {
+    uint32_t u;
+    std::memcpy(&u, &v, 4);
+    const uint16_t sign = uint16_t((u >> 16) & 0x8000u);
+    const uint32_t mag = u & 0x7fffffffu;
+    if (mag >= 0x7f800000u) return uint16_t(sign | 0x7c00u | (mag > 0x7f800000u ? 0x200u : 0u));   // inf / nan
+    if (mag >= 0x477ff000u) return uint16_t(sign | 0x7c00u);   // rounds to 65520 or more: infinity
+    if (mag < 0x33000001u) return sign;                        // at most half the smallest subnormal: zero
+    int32_t exp = int32_t(mag >> 23) - 127;
+    uint32_t man = (mag & 0x7fffffu) | 0x800000u;              // 24 significant bits
+    // binary16 keeps 11 significant bits of a normal number, fewer below 2^-14
+    const int shift = exp >= -14 ? 13 : 13 + (-14 - exp);
+    const uint32_t kept = man >> shift, rest = man & ((1u << shift) - 1u), half = 1u << (shift - 1);
+    uint32_t r = kept + uint32_t(rest > half || (rest == half && (kept & 1u)));
+    // normal: r carries the implicit bit at position 10, so adding the biased exponent minus one
+    // lets a carry out of the mantissa bump the exponent; subnormal: r is the mantissa itself
+    const uint32_t bits = exp >= -14 ? (uint32_t(exp + 15 - 1) << 10) + r : r;
+    return uint16_t(sign | bits);
+}
+
 }  // namespace
 
 int main(int argc, char** argv) {
@@ -82,7 +103,8 @@ int main(int argc, char** argv) {
     }
     if (c.elem_bytes == 2) {
         std::vector<uint16_t> elems(dZ);
-        for (uint64_t i = 0; i < dZ; ++i) elems[i] = to_bf16(host[i]);   // main.cu:59-62
+        const bool f16 = c.torch_dtype == KLEOS_DTYPE_FP16;
+        for (uint64_t i = 0; i < dZ; ++i) elems[i] = f16 ? to_f16(host[i]) : to_bf16(host[i]);   // main.cu:59-62
         HIP_OK(hipMemcpy(p, elems.data(), dZ * 2, hipMemcpyHostToDevice));
     } else {
         HIP_OK(hipMemcpy(p, host.data(), dZ * 4, hipMemcpyHostToDevice));
@@ -91,6 +113,35 @@ int main(int argc, char** argv) {
     kleos::moe::forwardHostBench<32, 32>(p, p + dZ * c.elem_bytes, timed);   // main.cu:68
     std::printf("epRank: %u took %.2fms\n", unsigned(rank), timed);         // main.cu:69
     HIP_OK(hipPeekAtLastError());
+    if (std::getenv("KLEOS_MAIN_CHECK")) {
+        // not in the reference's driver: the activations as the device holds them, decoded from the
+        // configured Element type, must still be the N(0, 5) sample that was drawn on the host
+        const uint64_t n = uint64_t(c.S) * c.H;
+        std::vector<char> raw(n * c.elem_bytes);
+        HIP_OK(hipMemcpy(raw.data(), p + c.off_x * c.elem_bytes, raw.size(), hipMemcpyDeviceToHost));
+        double sum = 0.0, sq = 0.0, err = 0.0;
+        for (uint64_t i = 0; i < n; ++i) {
+            float v;
+            if (c.elem_bytes == 4) {
+                std::memcpy(&v, &raw[i * 4], 4);
+            } else {
+                uint16_t h;
+                std::memcpy(&h, &raw[i * 2], 2);
+                if (c.torch_dtype == KLEOS_DTYPE_FP16) {
+                    const int e = (h >> 10) & 31, m = h & 1023;
+                    v = e == 0 ? std::ldexp(float(m), -24) : (e == 31 ? INFINITY : std::ldexp(float(m | 1024), e - 25));
+                    if (h & 0x8000u) v = -v;
+                } else {
+                    const uint32_t u = uint32_t(h) << 16;
+                    std::memcpy(&v, &u, 4);
+                }
+            }
+            sum += v; sq += double(v) * v;
+            err = std::fmax(err, std::fabs(double(v) - host[c.off_x + i]) / (std::fabs(host[c.off_x + i]) + 1e-3));
+        }
+        std::printf("device x: mean %.4f std %.4f max relative conversion error %.5f\n", sum / double(n),
+                    std::sqrt(sq / double(n)), err);
+    }
     kleos::finalize();
     HIP_OK(hipFree(p));
     return 0;

@@ -78,6 +78,27 @@ def measure_throughput(trials: int = 16) -> dict:
     return {"median_ms": float(ms.value), "throughput": float(thr.value)}
 
 
+def measure_throughput_output(derived, trials: int = 4) -> dict:
+    """The same probe, with its result y[pEC, H] copied back as raw Element words (uint16 for the
+    16-bit Elements, float32 otherwise)."""
+    ms = C.c_float(0.0)
+    thr = C.c_float(0.0)
+    y = np.empty((derived.pEC, derived.H), dtype=np.float32 if derived.elem_bytes == 4 else np.uint16)
+    _capi.check(_capi.lib().kleos_measure_throughput_output(int(trials), C.byref(ms), C.byref(thr), y.ctypes.data,
+                                                            y.nbytes))
+    return {"median_ms": float(ms.value), "throughput": float(thr.value), "y": y}
+
+
+def debug_set_wait_ticks(ticks: int) -> None:
+    """Bound of every wait inside the persistent kernel, in ticks of the 100 MHz device clock (0: default, 3 s)."""
+    _capi.check(_capi.lib().kleos_debug_set_wait_ticks(int(ticks)))
+
+
+def debug_skip_launch_number() -> None:
+    """Counts a persistent launch that never ran, so that the next one runs into its wait limit."""
+    _capi.check(_capi.lib().kleos_debug_skip_launch_number())
+
+
 def gate_loss(n_experts: int) -> dict:
     """Training mode: loss, mean probability [E] and mean routed count [E] of the last forward."""
     loss = C.c_float(0.0)

@@ -22,11 +22,36 @@ sys.path.insert(0, ROOT)
 PEAK_BF16_TFLOPS = 2500.0     # MI355X dense bf16 MFMA
 PEAK_FP32_TFLOPS = 157.3
 PEAK_HBM_GBS = 8000.0
-# HBM bytes per launch of the persistent kernel, from the two rocprofv3 --pmc passes (FETCH_SIZE,
-# WRITE_SIZE, each scaled by what the counter reads for a 1 GiB copy) summarised in
-# profiles/fused_kernel_headline_e64_zipf_hbm_traffic.txt. Counters cannot be read inside a timed
-# run, so the figure is carried here; --traffic-bytes overrides it after a new pair of passes.
-MEASURED_TRAFFIC_BYTES = {"headline_e64_zipf": 1.4306e9}
+
+
+def source_fingerprint() -> str:
+    """First 16 hex digits of the SHA-256 over the library's device and host sources: what a
+    committed counter summary was measured on."""
+    import hashlib
+    csrc = os.path.join(ROOT, "aristos_amd", "csrc")
+    h = hashlib.sha256()
+    for name in sorted(os.listdir(csrc)):
+        if name.endswith((".hip", ".hpp", ".cpp")):
+            with open(os.path.join(csrc, name), "rb") as f:
+                h.update(name.encode() + b"\0" + f.read())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic(workload: str):
+    """HBM bytes per launch of the persistent kernel as the committed rocprofv3 summary of this
+    workload states them (FETCH_SIZE and WRITE_SIZE passes, each scaled by what the counter reads
+    for a copy of known size): counters cannot be read inside a timed run. Returns (bytes or None,
+    whether the summary was made from the sources this run uses)."""
+    import re
+    path = os.path.join(ROOT, "profiles", f"fused_kernel_{workload}_hbm_traffic.txt")
+    if not os.path.exists(path):
+        return None, None
+    text = open(path).read()
+    m = re.search(r"=\s*([0-9.]+) GB of HBM traffic per launch", text)
+    if not m:
+        return None, None
+    fp = re.search(r"source fingerprint:\s*([0-9a-f]{16})", text)
+    return float(m.group(1)) * 1e9, bool(fp and fp.group(1) == source_fingerprint())
 
 
 def main() -> int:
@@ -42,12 +67,13 @@ def main() -> int:
     ap.add_argument("--calib-copy-mib", type=int, default=0,
                     help="also run one device-to-device copy of this many MiB before the timed region "
                          "(a kernel of known traffic to scale rocprofv3 FETCH_SIZE / WRITE_SIZE by)")
-    ap.add_argument("--traffic-bytes", type=float, default=None,
-                    help="measured HBM bytes per launch of the persistent kernel (from the rocprofv3 --pmc runs "
-                         "recorded under profiles/), reported as roofline.traffic")
+    ap.add_argument("--print-fingerprint", action="store_true",
+                    help="print the fingerprint of the library sources (recorded in the counter summaries) and exit")
     args = ap.parse_args()
-    if args.traffic_bytes is None:
-        args.traffic_bytes = MEASURED_TRAFFIC_BYTES.get(args.workload)
+    if args.print_fingerprint:
+        print(source_fingerprint())
+        return 0
+    traffic_bytes, traffic_current = measured_traffic(args.workload)
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures the single-GPU path (expert-parallel degree 1) only; run it with --gpus 1",
               file=sys.stderr)
@@ -135,6 +161,17 @@ def main() -> int:
         "combine_hbm_gbs": round((kept * d.H * eb + d.S * d.H * eb) / (ph["combine"] * 1e-3) / 1e9, 1) if ph["combine"] > 0 else None,
     }
 
+    # the expert phase alone (both projections of every expert, inside the persistent launch):
+    # weights once + the gathered activation rows, against both roofs
+    ex_bytes = float(2 * n_active * d.H * d.I * eb + kept * d.H * eb)
+    experts = None
+    if ex_ms > 0:
+        ex_gbs = ex_bytes / (ex_ms * 1e-3) / 1e9
+        ex_tf = flops_expert / (ex_ms * 1e-3) / 1e12
+        experts = {"ms": round(ex_ms, 4), "algorithmic_bytes": ex_bytes, "flops": flops_expert,
+                   "hbm": {"achieved": round(ex_gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(ex_gbs / PEAK_HBM_GBS, 4)},
+                   "mfma": {"achieved": round(ex_tf, 2), "peak": peak, "unit": "TFLOP/s", "frac": round(ex_tf / peak, 4)}}
+
     cpu = None
     if not args.no_cpu_baseline:
         cpu = cpu_baseline(w, iP, d, kept)
@@ -159,7 +196,7 @@ def main() -> int:
                    "expert_schedule": schedule + " (KLEOS_SCHEDULE_AUTO)"},
         "tokens_per_s": round(d.S / (wall_ms * 1e-3), 1),
         "event_ms_per_step": round(ev_ms, 5),
-        "roofline": roofline(flops_layer, hbm_bytes, ev_ms, peak, args.traffic_bytes),
+        "roofline": roofline(flops_layer, hbm_bytes, ev_ms, peak, traffic_bytes, traffic_current, experts),
         "fused_phases": fused_phases,
         "phased_mode": phases,
         "cpu_baseline": cpu,
@@ -168,7 +205,7 @@ def main() -> int:
     return 0
 
 
-def roofline(flops, hbm_bytes, ev_ms, mfma_peak, traffic):
+def roofline(flops, hbm_bytes, ev_ms, mfma_peak, traffic, traffic_current, experts):
     """The roof that binds the launch: below the ridge (peak FLOP/s / peak B/s) the algorithmic
     bytes cannot move faster than HBM, above it the FLOPs cannot run faster than the matrix cores.
     Both fractions are reported; `bound`, `achieved`, `peak`, `frac` describe the binding one."""
@@ -177,7 +214,7 @@ def roofline(flops, hbm_bytes, ev_ms, mfma_peak, traffic):
     tflops = flops / sec / 1e12
     intensity = flops / hbm_bytes
     ridge = mfma_peak * 1e12 / (PEAK_HBM_GBS * 1e9)
-    common = {"traffic": traffic, "kernel": "fused_kernel (whole layer: gate + slots + expert GEMMs + combine)",
+    common = {"traffic": traffic, "traffic_measured_on_these_sources": traffic_current, "experts": experts, "kernel": "fused_kernel (whole layer: gate + slots + expert GEMMs + combine)",
               "flops_per_launch": flops, "algorithmic_bytes_per_launch": hbm_bytes,
               "intensity_flop_per_byte": round(intensity, 1), "ridge_flop_per_byte": round(ridge, 1),
               "hbm": {"achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4)},

@@ -116,7 +116,15 @@ int kleos_get_config(kleos_config_t* cfg);
  * oP: device pointer, packed Elements  gateOut[S,PX] | moeOut[S,H]
  * Asynchronous on the library stream (the reference launches on kleosStream, types.cuh:1013); the
  * output is valid after kleos_stream_synchronize(). No host-side reset is needed between calls.
- * E == 1 runs the dense FFN (moe.cuh:197-204).
+ * E == 1 runs the dense FFN (moe.cuh:197-204) ON THE SAME PACKED LAYOUT as every other expert
+ * count: iP still carries the gate-weight block Wg[64,H] between x and Wup, and oP still starts
+ * with gateOut[S,64] (all ones in column 0), i.e. off_w_up = S*H + 64*H and off_moe_out = S*64,
+ * in_elems = S*H + 64*H + 2*I*H + I + H, out_elems = S*64 + S*H (kleos_get_config reports them).
+ * This is the layout the reference's driver packs for any E (csrc/main.cu:23-30). It is NOT the
+ * layout the reference's fffn kernel reads, iP = A | B1 | B2 | D1 | D2 and oP = C with no gate
+ * blocks (csrc/include/kleos/moe/fffn.cuh:43-49): the reference's driver and its fffn disagree with
+ * each other, and this library follows the driver. A caller that packs the fffn way must insert
+ * the 64*H gate block (any finite values) and read the result S*64 Elements into oP.
  */
 int kleos_moe_forward(const void* iP, void* oP);
 /*
@@ -197,6 +205,14 @@ int kleos_scheduler_stats(double stats[6]);
  * (experts per millisecond), the figure the reference stores in WorkerAttribute::throughput. Allocates
  * and frees its own operands; the context's state is untouched. */
 int kleos_measure_throughput(uint32_t trials, float* median_ms, float* throughput);
+/* The same probe, which also copies the first y_bytes of its result y[pEC, H] (Elements, row-major)
+ * to host memory before it frees its operands. The probe fills x, both weight matrices and both
+ * bias vectors with the byte 0x3c, so every Element has one value v (bf16 0.01147, fp16 1.0586,
+ * fp32 0.011489) and every result element is Element(I * Element(act(H*v*v + v)) * v + v): what the
+ * reference's probe computes is never looked at either (throughput.cuh:104-170 times the kernel of
+ * moe/expert.cuh:203-372), this lets a test check the launch geometry of the probe. */
+int kleos_measure_throughput_output(uint32_t trials, float* median_ms, float* throughput, void* y_host,
+                                    size_t y_bytes);
 /* Training mode (is_training: 1): the load-balancing loss of the gate of the most recent forward,
  * which the reference leaves in its bookkeeping arena (gML, gMeC, gL; csrc/include/kleos/types.cuh:
  * 940-958, computed at moe/gate.cuh:608-635, 700-705, 763-773): mean_prob[e] = mean over the tokens
@@ -211,6 +227,18 @@ int kleos_gate_loss(float* loss, float* mean_prob, float* mean_count);
  * [5] expert tiles done, [6] past barrier 3, [7] combine done. *n_workgroups receives the size of
  * the launch. */
 int kleos_phase_stamps(unsigned long long* stamps, uint32_t max_workgroups, uint32_t* n_workgroups);
+
+/* ---- failure handling of the persistent launch (no counterpart in the reference, whose waits are
+ * unbounded) ---- */
+/* Every wait inside the persistent kernel (grid barriers, row-block readiness) gives up after this
+ * many ticks of the device's 100 MHz wall clock (default 300 000 000 = 3 s; 0 restores the default):
+ * the grid always drains, the synchronising call that follows returns KLEOS_EHIP, and the library
+ * resets its scheduler counters so that the next forward behaves as on a fresh context. */
+int kleos_debug_set_wait_ticks(unsigned long long ticks);
+/* Makes the library count one persistent launch that never ran: the barrier counters then lag what
+ * the next launch expects, every barrier of that launch runs into its time limit, and the launch
+ * reports the expiry. For tests of the recovery path (with a small tick limit set first). */
+int kleos_debug_skip_launch_number(void);
 
 /* ---- errors --------------------------------------------------------------------------------- */
 /* Replaces the KLEOS_CHECK_CUDA / KLEOS_ASSERT message conventions (csrc/include/kleos/debug.cuh:

@@ -104,3 +104,20 @@ def test_json_round_trip(tmp_path):
     p = tmp_path / "c.json"
     p.write_text(cfg.to_json_text())
     assert ka.KleosConfig.from_json_file(str(p)) == cfg
+
+
+def test_single_expert_keeps_the_packed_moe_layout():
+    """E == 1 runs the dense FFN on the layout the reference's driver packs for every expert count
+    (csrc/main.cu:23-30: a 64-row gate-weight block after x, a 64-column gateOut block before the
+    result), not on the A | B1 | B2 | D1 | D2 -> C layout of the reference's fffn kernel
+    (csrc/include/kleos/moe/fffn.cuh:43-49). The offsets a caller needs are pinned here."""
+    S, H, I = 256, 128, 192
+    d = ka.KleosConfig(sequence_len=S, hidden_size=H, intermediate_size=I, num_experts=1, expert_top_k=1).derive()
+    assert (d.E, d.PX, d.k) == (1, 64, 1)
+    assert d.off_x == 0 and d.off_gate_w == S * H
+    assert d.off_w_up == S * H + 64 * H              # fffn would put B1 at S * H
+    assert d.off_w_down == d.off_w_up + I * H
+    assert d.off_b_up == d.off_w_down + H * I and d.off_b_down == d.off_b_up + I
+    assert d.in_elems == S * H + 64 * H + 2 * I * H + I + H
+    assert d.off_gate_out == 0 and d.off_moe_out == S * 64   # fffn would put C at 0
+    assert d.out_elems == S * 64 + S * H

@@ -472,21 +472,73 @@ def test_gate_loss_needs_training_mode():
 
 
 # ------------------------------------------------------------------ the reference's driver, on this library
-def test_cpp_driver_prints_the_reference_line(tmp_path):
+@pytest.mark.parametrize("dt", [2, 3, 0], ids=["bf16", "fp16", "fp32"])
+def test_cpp_driver_prints_the_reference_line(tmp_path, dt):
     """csrc/kleos_main is the equivalent of the reference's runOS() (csrc/main.cu:13-73): it reads a
-    kleos_config.json, fills the packed buffers on the host, runs forwardHostBench<32,32> through
-    kleos.hpp and prints `epRank: 0 took X ms`."""
+    kleos_config.json, fills the packed buffers on the host, converts them to Element (main.cu:59-62),
+    runs forwardHostBench<32,32> through kleos.hpp and prints `epRank: 0 took X ms`. With
+    KLEOS_MAIN_CHECK set it also reports how many output Elements are not finite: inputs converted
+    to the wrong 16-bit format (N(0, 5) values read as the other format) overflow at once."""
     import re
     import subprocess
     from aristos_amd import build
     if not os.path.exists(build.DRIVER_PATH):
         pytest.skip("the C++ driver is not built")
     cfg = tmp_path / "kleos_config.json"
-    cfg.write_text(_keys(1024, 256, 256, 16, 2).to_json_text())
-    r = subprocess.run([build.DRIVER_PATH, str(cfg)], capture_output=True, text=True, timeout=120)
+    cfg.write_text(_keys(512, 128, 128, 16, 2, dt=dt).to_json_text())
+    r = subprocess.run([build.DRIVER_PATH, str(cfg)], capture_output=True, text=True, timeout=120,
+                       env={**os.environ, "KLEOS_MAIN_CHECK": "1"})
     assert r.returncode == 0, r.stderr
     m = re.search(r"epRank: 0 took ([0-9.]+)\s*ms", r.stdout)
     assert m and float(m.group(1)) > 0, r.stdout
+    m = re.search(r"device x: mean (\S+) std (\S+) max relative conversion error (\S+)", r.stdout)
+    assert m, r.stdout
+    assert abs(float(m.group(1))) < 0.1 and abs(float(m.group(2)) - 5.0) < 0.1
+    assert float(m.group(3)) <= {2: 2.0 ** -8, 3: 2.0 ** -10, 0: 0.0}[dt]
+
+
+def _bytes_3c_value(dt):
+    """The value of an Element whose bytes are all 0x3c."""
+    if dt == 0:
+        return float(np.frombuffer(b"\x3c" * 4, np.float32)[0])
+    bits = np.array([0x3c3c], np.uint16)
+    return float(bits.view(np.float16)[0]) if dt == 3 else float(moe_ref.bf16_bits_to_f32(bits)[0])
+
+
+@pytest.mark.parametrize("dt,act,S,H,I,E", [(2, 0, 2048, 2048, 2048, 16), (2, 1, 1024, 256, 512, 8),
+                                            (3, 0, 1024, 128, 256, 8), (0, 1, 512, 128, 192, 4),
+                                            (2, 0, 8192, 256, 512, 2)])
+def test_throughput_probe_result(dt, act, S, H, I, E):
+    """The probe's operands are all one value v (every byte 0x3c), so every element of its result is
+    Element(I * Element(act(H v^2 + v)) * v + v), with the rounding points of the expert FFN
+    (processor.cuh:475, gemm.cuh:22-31). A wrong grid, a wrong capacity or a skipped tile of the
+    probe's E = 1, S = pEC launch leaves elements that differ."""
+    import math
+    keys = _keys(S, H, I, E, 2, act=act, dt=dt)
+    c = moe_ref.cfg_from_keys(keys)
+    d = ka.initialize(keys)
+    try:
+        r = ka.moe.measure_throughput_output(d, trials=3)
+    finally:
+        ka.finalize()
+    assert r["median_ms"] > 0 and r["y"].shape == (d.pEC, H)
+    v = _bytes_3c_value(dt)
+    pre = H * v * v + v
+    h1 = 0.5 * pre * (1.0 + math.erf(pre / math.sqrt(2.0))) if act == 1 else max(pre, 0.0)
+    def to_elem(val):
+        a = np.array([val], np.float32)
+        if dt == 0:
+            return float(a[0])
+        if dt == 3:
+            return float(a.astype(np.float16)[0])
+        return float(moe_ref.bf16_bits_to_f32(moe_ref.f32_to_bf16_bits(a))[0])
+    expect = to_elem(I * to_elem(h1) * v + v)
+    got = moe_ref.elems_to_f32(r["y"].ravel(), c).reshape(d.pEC, H)
+    # fp32 accumulation of equal terms in the matrix core's order against one multiplication: far
+    # below one rounding step of a 16-bit Element, a few ulp in fp32
+    tol = {0: 2e-6, 2: 2.0 ** -8, 3: 2.0 ** -11}[dt] * abs(expect)
+    assert np.isfinite(got).all()
+    assert np.abs(got - expect).max() <= tol, (expect, got.min(), got.max())
 
 
 def test_throughput_probe_leaves_the_context_alone():
@@ -508,5 +560,46 @@ def test_throughput_probe_leaves_the_context_alone():
         ka.moe.forward_host(iP, oP)
         ka.moe.stream_synchronize()
         np.testing.assert_array_equal(_out_to_np(c, oP), before)
+    finally:
+        ka.finalize()
+
+
+# ------------------------------------------------------------------ failure handling
+@pytest.mark.parametrize("schedule", [ka.SCHEDULE_DYNAMIC, ka.SCHEDULE_STATIC], ids=["dynamic", "static"])
+def test_context_recovers_after_an_expired_wait(schedule):
+    """A persistent launch whose grid barriers can never be satisfied (the host counts a launch that
+    never ran, so the monotonic arrival counters lag their targets) runs into the wait limit at every
+    barrier, drains, and is reported by the next synchronising call. The library then resets its
+    scheduler state: later forwards on the same context are bit-identical to a fresh context's.
+    The limit is lowered to 0.2 ms first; every kernel exits normally."""
+    keys = _keys(1024, 256, 256, 16, 2)
+    c = moe_ref.cfg_from_keys(keys)
+    x, wg, w_up, w_down, *_ = random_layer(c, seed=61, w_std=0.06)
+    iP = _to_device(c, pack_inputs(c, x, wg, w_up, w_down))
+    _, fresh, vf = run_gpu(keys, iP, (ka.MODE_FUSED, schedule))
+    fresh = _out_to_np(c, fresh)
+    d = ka.initialize(keys)
+    try:
+        _apply((ka.MODE_FUSED, schedule))
+        oP = synth.alloc_outputs(d)
+        ka.moe.forward_host(iP, oP)
+        ka.moe.forward_host(iP, oP)
+        ka.moe.stream_synchronize()
+        np.testing.assert_array_equal(_out_to_np(c, oP), fresh)
+        ka.moe.debug_set_wait_ticks(20000)          # 0.2 ms
+        ka.moe.debug_skip_launch_number()
+        ka.moe.forward_host(iP, oP)
+        with pytest.raises(ka.KleosError) as ei:
+            ka.moe.stream_synchronize()
+        assert ei.value.code == ka._capi.KLEOS_EHIP and "expired" in ei.value.message
+        ka.moe.debug_set_wait_ticks(0)
+        for _ in range(3):
+            oP.fill_(float("nan"))
+            torch.cuda.synchronize()
+            ka.moe.forward_host(iP, oP)
+            ka.moe.stream_synchronize()
+            np.testing.assert_array_equal(_out_to_np(c, oP), fresh)
+        v = ka.moe.debug_views(d)
+        np.testing.assert_array_equal(v["topk_slot"], vf["topk_slot"])
     finally:
         ka.finalize()
