@@ -8,6 +8,7 @@
 #include <algorithm>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <vector>
 
 #include "common.hpp"
@@ -107,21 +108,55 @@ int require_ctx(const char* who) {
     return KLEOS_OK;
 }
 
-LayerParams bind(const Context& c, const void* iP, void* oP) {
-    LayerParams p = c.base;
-    const size_t eb = c.cfg.elem_bytes;
+// The caller's packed buffers, sliced as moe.cuh:92-98.
+void bind_buffers(LayerParams& p, const kleos_config_t& cfg, const void* iP, void* oP) {
+    const size_t eb = cfg.elem_bytes;
     const char* in = static_cast<const char*>(iP);
     char* out = static_cast<char*>(oP);
-    // moe.cuh:92-98
-    p.x = in + c.cfg.off_x * eb;
-    p.wg = in + c.cfg.off_gate_w * eb;
-    p.w_up = in + c.cfg.off_w_up * eb;
-    p.w_down = in + c.cfg.off_w_down * eb;
-    p.b_up = in + c.cfg.off_b_up * eb;
-    p.b_down = in + c.cfg.off_b_down * eb;
-    p.gate_out = out + c.cfg.off_gate_out * eb;
-    p.moe_out = out + c.cfg.off_moe_out * eb;
+    p.x = in + cfg.off_x * eb;
+    p.wg = in + cfg.off_gate_w * eb;
+    p.w_up = in + cfg.off_w_up * eb;
+    p.w_down = in + cfg.off_w_down * eb;
+    p.b_up = in + cfg.off_b_up * eb;
+    p.b_down = in + cfg.off_b_down * eb;
+    p.gate_out = out + cfg.off_gate_out * eb;
+    p.moe_out = out + cfg.off_moe_out * eb;
+}
+
+LayerParams bind(const Context& c, const void* iP, void* oP) {
+    LayerParams p = c.base;
+    bind_buffers(p, c.cfg, iP, oP);
     return p;
+}
+
+// The configuration part of the kernel parameters (a derived configuration).
+void params_from_config(LayerParams& p, const kleos_config_t& cfg) {
+    p.S = cfg.S; p.H = cfg.H; p.I = cfg.I; p.E = cfg.E; p.k = cfg.k; p.PX = cfg.PX;
+    p.EC = cfg.EC; p.cap_rows = cfg.cap_rows; p.act = cfg.hidden_act;
+    p.is_training = cfg.is_training;
+    p.n_gate_tiles = cfg.S / kGateTileTokens;
+    p.n_super = (p.n_gate_tiles + kSuperTiles - 1) / kSuperTiles;
+    p.wait_ticks = kDefaultWaitTicks;
+}
+
+// The library-owned arrays of the kernel parameters, laid out in the memory at `a`.
+void params_from_arena(LayerParams& p, char* a, const ArenaLayout& L) {
+    p.logits = reinterpret_cast<float*>(a + L.logits);
+    p.topk_expert = reinterpret_cast<int32_t*>(a + L.topk_expert);
+    p.topk_prob = reinterpret_cast<float*>(a + L.topk_prob);
+    p.combine_den = reinterpret_cast<float*>(a + L.combine_den);
+    p.topk_slot = reinterpret_cast<int32_t*>(a + L.topk_slot);
+    p.tile_count = reinterpret_cast<uint32_t*>(a + L.tile_count);
+    p.super_count = reinterpret_cast<uint32_t*>(a + L.super_count);
+    p.expert_count = reinterpret_cast<uint32_t*>(a + L.expert_count);
+    p.slot_token = reinterpret_cast<int32_t*>(a + L.slot_token);
+    p.tile_prob = reinterpret_cast<float*>(a + L.tile_prob);
+    p.super_prob = reinterpret_cast<float*>(a + L.super_prob);
+    p.gate_loss = reinterpret_cast<float*>(a + L.gate_loss);
+    p.h1 = a + L.h1;
+    p.y = a + L.y;
+    p.sched = reinterpret_cast<uint32_t*>(a + L.sched);
+    p.stamps = reinterpret_cast<unsigned long long*>(a + L.stamps);
 }
 
 // Enqueues one forward. When ev is non-null (phased mode) it receives 6 recorded events that
@@ -189,36 +224,15 @@ extern "C" int kleos_initialize_cfg(const kleos_config_t* user_cfg) {
     KLEOS_HIP_BAIL(hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking));
 
     LayerParams& p = c->base;
-    p.S = cfg.S; p.H = cfg.H; p.I = cfg.I; p.E = cfg.E; p.k = cfg.k; p.PX = cfg.PX;
-    p.EC = cfg.EC; p.cap_rows = cfg.cap_rows; p.act = cfg.hidden_act;
-    p.is_training = cfg.is_training;
-    p.n_gate_tiles = cfg.S / kGateTileTokens;
-    p.n_super = (p.n_gate_tiles + kSuperTiles - 1) / kSuperTiles;
+    params_from_config(p, cfg);
     const ArenaLayout L = layout_arena(cfg, p.n_gate_tiles, p.n_super);
     KLEOS_HIP_BAIL(hipMalloc(reinterpret_cast<void**>(&c->arena), L.total));
     c->arena_bytes = L.total;
     c->zero_begin = L.zero_begin;
     c->zero_end = L.zero_end;
-    p.wait_ticks = kDefaultWaitTicks;
     KLEOS_HIP_BAIL(hipMemsetAsync(c->arena + L.zero_begin, 0, L.zero_end - L.zero_begin, c->stream));
     KLEOS_HIP_BAIL(hipStreamSynchronize(c->stream));
-    char* a = c->arena;
-    p.logits = reinterpret_cast<float*>(a + L.logits);
-    p.topk_expert = reinterpret_cast<int32_t*>(a + L.topk_expert);
-    p.topk_prob = reinterpret_cast<float*>(a + L.topk_prob);
-    p.combine_den = reinterpret_cast<float*>(a + L.combine_den);
-    p.topk_slot = reinterpret_cast<int32_t*>(a + L.topk_slot);
-    p.tile_count = reinterpret_cast<uint32_t*>(a + L.tile_count);
-    p.super_count = reinterpret_cast<uint32_t*>(a + L.super_count);
-    p.expert_count = reinterpret_cast<uint32_t*>(a + L.expert_count);
-    p.slot_token = reinterpret_cast<int32_t*>(a + L.slot_token);
-    p.tile_prob = reinterpret_cast<float*>(a + L.tile_prob);
-    p.super_prob = reinterpret_cast<float*>(a + L.super_prob);
-    p.gate_loss = reinterpret_cast<float*>(a + L.gate_loss);
-    p.h1 = a + L.h1;
-    p.y = a + L.y;
-    p.sched = reinterpret_cast<uint32_t*>(a + L.sched);
-    p.stamps = reinterpret_cast<unsigned long long*>(a + L.stamps);
+    params_from_arena(p, c->arena, L);
     KLEOS_HIP_BAIL(plan_fused(p, int(cfg.torch_dtype), c->num_cus, &c->plan));
     if (c->plan.nwg > kMaxWorkgroups) return bail(fail(KLEOS_EUNSUPPORTED, "persistent grid of %u workgroups exceeds %u", c->plan.nwg, kMaxWorkgroups));
 #undef KLEOS_HIP_BAIL
