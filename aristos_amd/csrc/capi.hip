@@ -186,10 +186,90 @@ int enqueue_forward(Context& c, const void* iP, void* oP, hipEvent_t* ev) {
     return KLEOS_OK;
 }
 
+// ---------------------------------------------------------------- the entry point that allocates nothing
+// Every library-owned array of a forward (routing tables, h1, y, scheduler counters, stamps) laid out
+// in a fixed array in device memory instead of an arena from hipMalloc. Every GPU the library runs
+// on holds its own copy of the array, at its own address, until the process ends.
+constexpr size_t kStaticScratchBytes = KLEOS_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+// What a device needs once: the address of its copy of `scratch` (in host code the array's name is
+// only a handle for hipGetSymbolAddress, never a device address) and its compute-unit count.
+struct DeviceSetup {
+    bool ready = false;
+    char* scratch_ptr = nullptr;
+    int num_cus = 0;
+    bool gfx950 = false;
+};
+constexpr int kMaxDevices = 64;
+DeviceSetup g_devices[kMaxDevices];
+std::mutex g_devices_mutex;
+
+// Looks the current device up (first call per device) or returns what was found then.
+int device_setup(const DeviceSetup** out) {
+    int dev = -1;
+    KLEOS_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return fail(KLEOS_EUNSUPPORTED, "device ordinal %d is beyond %d", dev, kMaxDevices);
+    std::lock_guard<std::mutex> lock(g_devices_mutex);
+    DeviceSetup& d = g_devices[dev];
+    if (!d.ready) {
+        void* ptr = nullptr;
+        KLEOS_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        if (!ptr) return fail(KLEOS_EHIP, "hipGetSymbolAddress returned a null address for the static scratch");
+        hipDeviceProp_t prop;
+        KLEOS_HIP(hipGetDeviceProperties(&prop, dev));
+        d.scratch_ptr = static_cast<char*>(ptr);
+        d.num_cus = prop.multiProcessorCount;
+        d.gfx950 = std::strncmp(prop.gcnArchName, "gfx950", 6) == 0;
+        d.ready = true;
+    }
+    *out = &d;
+    return KLEOS_OK;
+}
+
+__global__ __launch_bounds__(256) void zero_words_kernel(uint32_t* words, size_t n) {
+    for (size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += size_t(gridDim.x) * blockDim.x) words[i] = 0u;
+}
+
 }  // namespace
 }  // namespace kleos_amd
 
 using namespace kleos_amd;
+
+extern "C" int kleos_moe_forward_static_scratch(const kleos_config_t* user_cfg, const void* iP, void* oP, void* stream) {
+    if (!user_cfg) return fail(KLEOS_EINVAL, "kleos_moe_forward_static_scratch: null config");
+    if (!iP || !oP) return fail(KLEOS_EINVAL, "kleos_moe_forward_static_scratch: null buffer");
+    if ((reinterpret_cast<uintptr_t>(iP) | reinterpret_cast<uintptr_t>(oP)) & 15u)
+        return fail(KLEOS_EINVAL, "kleos_moe_forward_static_scratch: iP and oP must be 16-byte aligned");
+    kleos_config_t cfg = *user_cfg;
+    if (int rc = kleos_config_derive(&cfg)) return rc;
+    if (const char* why = unsupported_reason(cfg.E, cfg.k)) return fail(KLEOS_EUNSUPPORTED, "%s", why);
+    const DeviceSetup* dev = nullptr;
+    if (int rc = device_setup(&dev)) return rc;
+    if (!dev->gfx950) return fail(KLEOS_EUNSUPPORTED, "the current device is not gfx950: this library is built for MI355X only");
+    LayerParams p{};
+    params_from_config(p, cfg);
+    const ArenaLayout L = layout_arena(cfg, p.n_gate_tiles, p.n_super);
+    if (L.total > kStaticScratchBytes)
+        return fail(KLEOS_EUNSUPPORTED, "kleos_moe_forward_static_scratch: this configuration needs %zu bytes of library "
+                    "memory, the static scratch holds %zu; use kleos_initialize + kleos_moe_forward", L.total,
+                    kStaticScratchBytes);
+    params_from_arena(p, dev->scratch_ptr, L);
+    bind_buffers(p, cfg, iP, oP);
+    FusedPlan plan;
+    KLEOS_HIP(plan_fused(p, int(cfg.torch_dtype), dev->num_cus, &plan));
+    if (plan.nwg > kMaxWorkgroups) return fail(KLEOS_EUNSUPPORTED, "persistent grid of %u workgroups exceeds %u", plan.nwg, kMaxWorkgroups);
+    // The array keeps what the last call left, of whatever configuration: every counter goes back
+    // to zero (a fill kernel, which a stream capture records faithfully), and the launch runs as the
+    // first one of a fresh arena.
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const size_t words = (L.zero_end - L.zero_begin) / 4;
+    hipLaunchKernelGGL(zero_words_kernel, dim3(64), dim3(256), 0, s, reinterpret_cast<uint32_t*>(dev->scratch_ptr + L.zero_begin), words);
+    KLEOS_HIP(hipGetLastError());
+    p.epoch = 0;
+    KLEOS_HIP(launch_fused(p, plan, 0, KLEOS_SCHEDULE_AUTO, s));
+    return KLEOS_OK;
+}
 
 extern "C" int kleos_initialize_cfg(const kleos_config_t* user_cfg) {
     if (!user_cfg) return fail(KLEOS_EINVAL, "kleos_initialize_cfg: null config");
@@ -214,6 +294,11 @@ extern "C" int kleos_initialize_cfg(const kleos_config_t* user_cfg) {
                              hipGetErrorName(e_), hipGetErrorString(e_)));                      \
     } while (0)
     KLEOS_HIP_BAIL(hipGetDevice(&c->device));
+    {
+        // the address of this device's static scratch, for kleos_moe_forward_static_scratch
+        const DeviceSetup* dev = nullptr;
+        if (int rc = device_setup(&dev)) return bail(rc);
+    }
     hipDeviceProp_t prop;
     KLEOS_HIP_BAIL(hipGetDeviceProperties(&prop, c->device));
     c->num_cus = prop.multiProcessorCount;

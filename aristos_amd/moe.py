@@ -32,6 +32,13 @@ def forward_host_bench(iP, oP, skip: int = 32, trials: int = 32) -> float:
     return float(ms.value)
 
 
+def forward_static_scratch(config, iP, oP, stream: int = 0) -> None:
+    """kleos_moe_forward_static_scratch: one forward of the layer `config` (a KleosConfig) that allocates
+    nothing, on `stream` (a hipStream_t as an integer; 0 = the default stream). Asynchronous."""
+    st = config.to_struct()
+    _capi.check(_capi.lib().kleos_moe_forward_static_scratch(C.byref(st), _ptr(iP), _ptr(oP), stream or None))
+
+
 def stream_synchronize() -> None:
     _capi.check(_capi.lib().kleos_stream_synchronize())
 

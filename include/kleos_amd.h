@@ -134,6 +134,26 @@ int kleos_moe_forward(const void* iP, void* oP);
  */
 int kleos_moe_forward_bench(const void* iP, void* oP, uint32_t skip, uint32_t trials,
                             float* ms_per_launch);
+/*
+ * No counterpart in the reference. For callers that cannot allocate device memory around a forward:
+ * code under HIP stream capture, tight serving loops, harnesses that forbid hipMalloc. The same
+ * forward as kleos_moe_forward (persistent launch, KLEOS_SCHEDULE_AUTO), but every library-owned array
+ * (routing tables, the activations between the projections, scheduler counters) lives in a fixed
+ * array of KLEOS_STATIC_SCRATCH_BYTES bytes in device memory that each GPU holds from the moment the
+ * library is loaded until the process ends. Needs no kleos_initialize and leaves an initialised
+ * context alone; calls no hipMalloc / hipFree or any other allocating routine.
+ *   cfg:    the JSON keys of the layer (derived fields are recomputed); a configuration whose arrays
+ *           do not fit the scratch is refused with KLEOS_EUNSUPPORTED (the message states both sizes)
+ *   iP, oP: as for kleos_moe_forward, on the current device
+ *   stream: a hipStream_t (NULL: the default stream); the call enqueues a fill kernel that clears the
+ *           counters, then the persistent kernel, and returns. The output is valid once the
+ *           stream has drained.
+ * All calls on one GPU share that GPU's array: calls that overlap on a GPU (two streams, two
+ * threads) race and give wrong results; calls on one stream are ordered and safe, whatever their
+ * configurations. An expired in-kernel wait (see kleos_debug_set_wait_ticks) is not reported here.
+ */
+#define KLEOS_STATIC_SCRATCH_BYTES (32u << 20)
+int kleos_moe_forward_static_scratch(const kleos_config_t* cfg, const void* iP, void* oP, void* stream);
 /* Blocks until everything queued on the library stream has finished
  * (cudaStreamSynchronize(kleosStream) in the reference's callers, csrc/main.cu:64-70). */
 int kleos_stream_synchronize(void);

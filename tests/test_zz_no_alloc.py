@@ -1,0 +1,107 @@
+"""kleos_moe_forward_static_scratch: the forward that allocates nothing (its library-owned arrays live
+in a fixed array in device memory) gives the bits of kleos_moe_forward, on calls in a row that share
+the array: a layer, then a smaller one of a different shape, then the first again."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+import aristos_amd as ka
+from aristos_amd import _capi, synth
+from helpers import pack_inputs, random_layer
+from oracle import moe_ref
+
+pytestmark = pytest.mark.gpu
+
+
+def _keys(S, H, I, E, k, dt=2, cf=1.0):
+    return ka.KleosConfig(capacity_factor=cf, drop_tokens=1, expert_top_k=k, hidden_act=0, hidden_size=H,
+                          intermediate_size=I, num_experts=E, sequence_len=S, mini_batch=1, torch_dtype=dt)
+
+
+def _device_inputs(keys, seed):
+    c = moe_ref.cfg_from_keys(keys)
+    x, wg, w_up, w_down, b_up, b_down = random_layer(c, seed=seed, w_std=0.08, bias_std=0.1)
+    wg[0] *= 2.5                                   # an expert that overflows: dropped tokens
+    if c.dtype == 2:
+        from np_restatement import round_bf16
+        wg = round_bf16(wg)
+    iP_np = pack_inputs(c, x, wg, w_up, w_down, b_up, b_down)
+    if c.dtype in (2, 3):
+        iP = torch.from_numpy(iP_np.view(np.int16)).cuda().view(torch.bfloat16 if c.dtype == 2 else torch.float16)
+    else:
+        iP = torch.from_numpy(iP_np).cuda()
+    return c, iP
+
+
+def _bits(c, oP):
+    return oP.view(torch.int16).cpu().numpy().copy() if c.dtype in (2, 3) else oP.cpu().numpy().copy()
+
+
+def _existing_entry_point(keys, iP):
+    d = ka.initialize(keys)
+    try:
+        oP = synth.alloc_outputs(d)
+        oP.fill_(float("nan"))
+        torch.cuda.synchronize()
+        ka.moe.forward_host(iP, oP)
+        ka.moe.stream_synchronize()
+        return d, oP
+    finally:
+        ka.finalize()
+
+
+def test_static_scratch_forward_matches_the_allocating_one():
+    big = _keys(1024, 256, 512, 16, 2)
+    small = _keys(256, 128, 128, 8, 2, cf=2.0)
+    small_f32 = _keys(128, 64, 64, 4, 1, dt=0)
+    cases = []
+    for keys, seed in ((big, 71), (small, 72), (small_f32, 73)):
+        c, iP = _device_inputs(keys, seed)
+        d, ref = _existing_entry_point(keys, iP)
+        cases.append((keys, c, d, iP, _bits(c, ref)))
+    assert not ka.is_initialized()
+    # calls in a row on the default stream, no context: big, small, smaller still (fp32), big again
+    for keys, c, d, iP, ref in (cases[0], cases[1], cases[2], cases[0], cases[1]):
+        oP = synth.alloc_outputs(d)
+        oP.fill_(float("nan"))
+        torch.cuda.synchronize()
+        ka.moe.forward_static_scratch(keys, iP, oP)
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(_bits(c, oP), ref)
+    # two calls queued back to back without a synchronisation in between share the array in order
+    (k0, c0, d0, i0, r0), (k1, c1, d1, i1, r1) = cases[0], cases[1]
+    o0, o1 = synth.alloc_outputs(d0), synth.alloc_outputs(d1)
+    torch.cuda.synchronize()
+    ka.moe.forward_static_scratch(k0, i0, o0)
+    ka.moe.forward_static_scratch(k1, i1, o1)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(_bits(c0, o0), r0)
+    np.testing.assert_array_equal(_bits(c1, o1), r1)
+    # an initialised context is left alone, and works beside it
+    d = ka.initialize(k1)
+    try:
+        oa, ob = synth.alloc_outputs(d1), synth.alloc_outputs(d0)
+        ka.moe.forward_host(i1, oa)
+        ka.moe.stream_synchronize()
+        ka.moe.forward_static_scratch(k0, i0, ob)
+        torch.cuda.synchronize()
+        ka.moe.forward_host(i1, oa)
+        ka.moe.stream_synchronize()
+        np.testing.assert_array_equal(_bits(c1, oa), r1)
+        np.testing.assert_array_equal(_bits(c0, ob), r0)
+    finally:
+        ka.finalize()
+
+
+def test_static_scratch_refuses_what_does_not_fit():
+    """The headline layer needs about 134 MB of library arrays: beyond the 32 MiB the scratch holds."""
+    keys = synth.WORKLOADS["headline_e64_zipf"].config
+    dummy = torch.zeros(64, dtype=torch.bfloat16, device="cuda")
+    st = keys.to_struct()
+    rc = _capi.lib().kleos_moe_forward_static_scratch(ctypes.byref(st), dummy.data_ptr(), dummy.data_ptr(), None)
+    assert rc == _capi.KLEOS_EUNSUPPORTED
+    msg = _capi.lib().kleos_last_error().decode()
+    assert "static scratch holds 33554432" in msg, msg
+    torch.cuda.synchronize()
