@@ -16,9 +16,14 @@ namespace kleos_amd {
 //
 // K is walked in slices of BK through a ring of LDS stages that the wavefronts fill with direct
 // global->LDS loads (global_load_lds_dwordx4: each lane names a 16-byte global source, the 64 lanes
-// of the instruction land in 1 KB of consecutive LDS). The loads of the next STAGES-1 slices are in
-// flight while a slice is multiplied, and never occupy a vector register. Rows of A are gathered
-// through the slot->token table by giving each lane its token's row address.
+// of the instruction land in 1 KB of consecutive LDS). They never occupy a vector register. Rows of
+// A are gathered through the slot->token table by giving each lane its token's row address.
+// Slice kt+STAGES-1 is requested at the start of slice kt, into the stage slice kt-1 was read from.
+// With two stages the loads can instead run two slices ahead (AHEAD2): slice kt+2 is requested
+// into the stage of slice kt as soon as every wavefront has read its last fragments of slice kt (a
+// second workgroup barrier per slice, placed before the last group of matrix instructions), so the
+// memory pipeline holds requests across the wait for slice kt+1 instead of running empty at
+// every slice boundary.
 //
 // LDS layout of a stage: rows of BK*2 bytes, 16-byte chunk c of row r stored at chunk position
 // c ^ swizzle(r). The LDS of gfx950 has 64 banks of 4 bytes and serves a 16-byte access of 16 lanes
@@ -134,11 +139,15 @@ __device__ __forceinline__ void epilogue16(const TileOut& t, f32x16 (&acc)[WN / 
     else epilogue16_act<E, WM, WN, WAVES_N, 2>(t, acc, stage_mem, bias_mem);
 }
 
-// ISSUE: over how many K steps of a slice the loads of the slice STAGES-1 ahead are issued.
 // STREAM_B: the weight rows are loaded with the non-temporal cache policy: read once (or by a
 // neighbour at the same moment), they pass through the L2 without displacing the activation rows
 // that are shared (7.0 against 6.4 TB/s on a read-only stream of this shape).
-template <typename E, int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES, int ISSUE, bool STREAM_B>
+// AHEAD2 (two stages only): the loads run two slices ahead, at the price of a second workgroup
+// barrier per slice. It pays where the weights stream from HBM and a slice's loads take longer than
+// its matrix work (headline shape: 301 against 315 us for the expert phase); where the matrix work
+// dominates the extra barrier costs more than the earlier loads bring (8-expert shape with hidden
+// size 4096: 4.22 against 4.03 ms).
+template <typename E, int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES, bool STREAM_B, bool AHEAD2>
 struct Gemm16 {
     typedef typename Elem16<E>::vec8 vec8;
     typedef typename Elem16<E>::vec4 vec4;
@@ -160,9 +169,8 @@ struct Gemm16 {
     static constexpr int kSliceK = BK;                             // values of K per slice
     static constexpr int kSteps = BK / 16;                         // matrix instructions consume 16 values of K
     static constexpr int kPanelRows = kEpiloguePanelRows;          // epilogue staging: 32 rows x 64 columns per wavefront
-    static constexpr int kIssueSteps = ISSUE;                      // K steps over which the next slice's loads are issued
-    static_assert(ISSUE >= 1 && ISSUE <= kSteps);
     static_assert(BK == 32 || BK == 64);
+    static_assert(!AHEAD2 || STAGES == 2);
     static_assert(STAGES >= 2 && STAGES <= 4);
     static_assert(WM % 32 == 0 && WN % 64 == 0);
     static_assert(BM % (kRowsPerLoad * kWaves) == 0 && BN % (kRowsPerLoad * kWaves) == 0);
@@ -189,8 +197,9 @@ struct Gemm16 {
 
     static __device__ __forceinline__ int stage_of(const Tile& t, uint32_t kt) { return (t.stage0 + kt) % STAGES; }
 
-    // part `part` of `parts` of the direct loads that bring K slice kt of the tile into its stage
-    static __device__ __forceinline__ void issue_part(const Tile& t, char* smem, uint32_t kt, int part, int parts) {
+    // the direct loads that bring K slice kt of the tile into its stage: activation rows first (they
+    // come from L2 and return early), then the weight rows
+    static __device__ __forceinline__ void issue_slice(const Tile& t, char* smem, uint32_t kt) {
         const int wave = threadIdx.x >> 6;
         char* sa = smem + stage_of(t, kt) * kStage;
         char* sb = sa + kABytes;
@@ -199,13 +208,11 @@ struct Gemm16 {
         const uint32_t k0 = slice * BK;
 #pragma unroll
         for (int i = 0; i < LA; ++i)
-            if (i * parts / LA == part)
-                __builtin_amdgcn_global_load_lds((global_cptr)(t.pa[i] + k0), (lds_ptr)(sa + 1024 * (wave + kWaves * i)), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((global_cptr)(t.pa[i] + k0), (lds_ptr)(sa + 1024 * (wave + kWaves * i)), 16, 0, 0);
 #pragma unroll
         for (int i = 0; i < LB; ++i)
-            if (i * parts / LB == part)
-                __builtin_amdgcn_global_load_lds((global_cptr)(t.pb[i] + k0), (lds_ptr)(sb + 1024 * (wave + kWaves * i)), 16, 0,
-                                                 STREAM_B ? kNonTemporal : 0);
+            __builtin_amdgcn_global_load_lds((global_cptr)(t.pb[i] + k0), (lds_ptr)(sb + 1024 * (wave + kWaves * i)), 16, 0,
+                                             STREAM_B ? kNonTemporal : 0);
     }
 
     // Per-lane source addresses, the load of the bias into LDS slot `bias_slot`, then the loads of
@@ -221,19 +228,26 @@ struct Gemm16 {
             const uint32_t n = uint32_t(lane) * 8 < g.n_valid ? uint32_t(lane) * 8 : 0u;
             __builtin_amdgcn_global_load_lds((global_cptr)(g.bias + n), (lds_ptr)(smem + kBiasOffset + bias_slot * kBiasBytes), 16, 0, 0);
         }
+        // The lane's source rows. The slot->token table was written earlier in the same launch,
+        // possibly on another XCD: device-coherent loads, all in flight together (an index is clamped
+        // to the table it points into, so that no value it could ever hold turns into an address
+        // outside the caller's buffer).
+        uint32_t src[LA];
 #pragma unroll
         for (int i = 0; i < LA; ++i) {
             const int row = kRowsPerLoad * (wave + kWaves * i) + ld_r;
-            const uint32_t r = row < int(g.m_valid) ? row : g.m_valid - 1;
-            // the slot->token table was written earlier in the same launch, possibly on another XCD
-            // (an index is clamped to the table it points into, so that no value it could ever
-            // hold turns into an address outside the caller's buffer)
-            uint32_t src = r;
-            if (g.a_row_index) {
-                src = uint32_t(load_coherent(g.a_row_index + r));
-                src = src < g.a_rows ? src : g.a_rows - 1;
-            }
-            t.pa[i] = g.a_base + size_t(src) * g.lda + ((ld_p ^ swizzle(row)) << 3);
+            src[i] = row < int(g.m_valid) ? row : g.m_valid - 1;
+        }
+        if (g.a_row_index) {
+#pragma unroll
+            for (int i = 0; i < LA; ++i) src[i] = uint32_t(load_coherent(g.a_row_index + src[i]));
+#pragma unroll
+            for (int i = 0; i < LA; ++i) src[i] = src[i] < g.a_rows ? src[i] : g.a_rows - 1;
+        }
+#pragma unroll
+        for (int i = 0; i < LA; ++i) {
+            const int row = kRowsPerLoad * (wave + kWaves * i) + ld_r;
+            t.pa[i] = g.a_base + size_t(src[i]) * g.lda + ((ld_p ^ swizzle(row)) << 3);
         }
 #pragma unroll
         for (int i = 0; i < LB; ++i) {
@@ -247,7 +261,7 @@ struct Gemm16 {
         t.act = g.act; t.stage0 = stage0; t.bias_slot = bias_slot;
 #pragma unroll
         for (int st = 0; st < STAGES - 1; ++st)
-            if (uint32_t(st) < t.k_tiles) issue_part(t, smem, st, 0, 1);
+            if (uint32_t(st) < t.k_tiles) issue_slice(t, smem, st);
     }
 
     static __device__ __forceinline__ void mainloop(const Tile& t, Acc& acc, char* smem) {
@@ -266,42 +280,68 @@ struct Gemm16 {
         const int rx = wm * WM + fr_row, rw = wn * WN + fr_row;
         const int base_x = rx * kRowBytes + ((fr_half ^ swizzle(rx)) << 4);
         const int base_w = kABytes + rw * kRowBytes + ((fr_half ^ swizzle(rw)) << 4);
-        for (uint32_t kt = 0; kt < t.k_tiles; ++kt) {
-            // This wavefront's loads of slice kt are complete once only those of the later slices
-            // already issued (STAGES-2 of them, fewer at the end of the tile) are outstanding.
-            const uint32_t later = t.k_tiles - 1 - kt;
-            if (STAGES >= 4 && later >= 2) wait_vmcnt<(STAGES >= 4 ? 2 : 0) * kLoadsPerSlice>();
-            else if (STAGES >= 3 && later >= 1) wait_vmcnt<(STAGES >= 3 ? 1 : 0) * kLoadsPerSlice>();
-            else wait_vmcnt<0>();
-            // every wavefront's share of slice kt is in LDS, and everyone has finished with the stage
-            // the next loads overwrite (slice kt-1, or the previous tile's epilogue staging)
+        // The operand fragments of K step ks+1 are read from LDS while the matrix core works on step ks.
+        vec8 fw[2][TN], fx[2][TM];
+        auto read_fragments = [&](const char* st, int ks) {
+#pragma unroll
+            for (int ni = 0; ni < TN; ++ni) fw[ks & 1][ni] = __builtin_bit_cast(vec8, load16(st + (base_w ^ (ks << 5)) + ni * 32 * kRowBytes));
+#pragma unroll
+            for (int mi = 0; mi < TM; ++mi) fx[ks & 1][mi] = __builtin_bit_cast(vec8, load16(st + (base_x ^ (ks << 5)) + mi * 32 * kRowBytes));
+        };
+        auto multiply = [&](int ks) {
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int ni = 0; ni < TN; ++ni)
+#pragma unroll
+                for (int mi = 0; mi < TM; ++mi)
+                    acc[ni][mi] = Elem16<E>::mfma32(fw[ks & 1][ni], fx[ks & 1][mi], acc[ni][mi]);
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        if constexpr (AHEAD2) {
+            // Slice 0 was requested by begin(). Every wavefront has left the previous tile's epilogue,
+            // which staged its output in the stage slice 1 goes to.
             asm volatile("s_barrier" ::: "memory");
-            // The loads of slice kt+STAGES-1 are spread over the K steps of this slice rather than
-            // issued in one burst, which would hold the wavefront in the address queue.
-            const uint32_t ahead = kt + STAGES - 1;
-            const bool more = ahead < t.k_tiles;
-            const char* st = smem + stage_of(t, kt) * kStage;
-            // The operand fragments of K step ks+1 are read from LDS while the matrix core works
-            // on step ks.
-            vec8 fw[2][TN], fx[2][TM];
-            auto read_fragments = [&](int ks) {
+            if (t.k_tiles > 1) issue_slice(t, smem, 1);
+            for (uint32_t kt = 0; kt < t.k_tiles; ++kt) {
+                // this wavefront's loads of slice kt are complete once only those of slice kt+1 are
+                // outstanding (the stores of the previous tile's epilogue are older than both)
+                if (kt + 1 < t.k_tiles) wait_vmcnt<kLoadsPerSlice>();
+                else wait_vmcnt<0>();
+                asm volatile("s_barrier" ::: "memory");   // every wavefront's share of slice kt is in LDS
+                const char* st = smem + stage_of(t, kt) * kStage;
+                read_fragments(st, 0);
 #pragma unroll
-                for (int ni = 0; ni < TN; ++ni) fw[ks & 1][ni] = __builtin_bit_cast(vec8, load16(st + (base_w ^ (ks << 5)) + ni * 32 * kRowBytes));
+                for (int ks = 0; ks < kSteps; ++ks) {
+                    if (ks + 1 < kSteps) read_fragments(st, ks + 1);
+                    if (ks == kSteps - 1 && kt + 2 < t.k_tiles) {
+                        // this wavefront's last reads of the stage have returned; once that holds for
+                        // every wavefront the stage takes slice kt+2
+                        __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0)
+                        asm volatile("s_barrier" ::: "memory");
+                        issue_slice(t, smem, kt + 2);
+                    }
+                    multiply(ks);
+                }
+            }
+        } else {
+            for (uint32_t kt = 0; kt < t.k_tiles; ++kt) {
+                // This wavefront's loads of slice kt are complete once only those of the later slices
+                // already issued (STAGES-2 of them, fewer at the end of the tile) are outstanding.
+                const uint32_t later = t.k_tiles - 1 - kt;
+                if (STAGES >= 4 && later >= 2) wait_vmcnt<(STAGES >= 4 ? 2 : 0) * kLoadsPerSlice>();
+                else if (STAGES >= 3 && later >= 1) wait_vmcnt<kLoadsPerSlice>();
+                else wait_vmcnt<0>();
+                // every wavefront's share of slice kt is in LDS, and everyone has finished with the stage
+                // the next loads overwrite (slice kt-1, or the previous tile's epilogue staging)
+                asm volatile("s_barrier" ::: "memory");
+                const char* st = smem + stage_of(t, kt) * kStage;
+                read_fragments(st, 0);
 #pragma unroll
-                for (int mi = 0; mi < TM; ++mi) fx[ks & 1][mi] = __builtin_bit_cast(vec8, load16(st + (base_x ^ (ks << 5)) + mi * 32 * kRowBytes));
-            };
-            read_fragments(0);
-#pragma unroll
-            for (int ks = 0; ks < kSteps; ++ks) {
-                if (ks + 1 < kSteps) read_fragments(ks + 1);
-                if (more && ks < kIssueSteps) issue_part(t, smem, ahead, ks, kIssueSteps);
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int ni = 0; ni < TN; ++ni)
-#pragma unroll
-                    for (int mi = 0; mi < TM; ++mi)
-                        acc[ni][mi] = Elem16<E>::mfma32(fw[ks & 1][ni], fx[ks & 1][mi], acc[ni][mi]);
-                __builtin_amdgcn_sched_barrier(0);
+                for (int ks = 0; ks < kSteps; ++ks) {
+                    if (ks + 1 < kSteps) read_fragments(st, ks + 1);
+                    if (ks == 0 && kt + STAGES - 1 < t.k_tiles) issue_slice(t, smem, kt + STAGES - 1);
+                    multiply(ks);
+                }
             }
         }
     }
