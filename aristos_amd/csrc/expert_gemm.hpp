@@ -39,10 +39,11 @@ namespace kleos_amd {
 //   begin()    per-lane source addresses + the loads of the bias and of the first STAGES-1 slices
 //   mainloop() all K slices
 //   finish()   bias, activation, rounding, transposition through LDS, coalesced stores
-// A workgroup calls begin() of its next tile between mainloop() and finish() of the current one,
-// so the next tile's first loads and its index look-ups travel while the epilogue runs: the stage
-// ring keeps turning across tiles, finish() stages its output in the one stage the next tile's
-// first loads do not touch (the stage of the last slice).
+// A workgroup calls finish() of a tile, then begin() of its next one: the stores enter the memory
+// pipeline ahead of the next tile's loads (measured: 2 % faster than the other order, in which the
+// stores queue behind a slice of loads and hold the wavefronts that issue them), and the stage ring
+// keeps turning across tiles (finish() stages its output in the stage of the last slice, which
+// every wavefront has left; begin() follows behind a workgroup barrier of the caller).
 // ------------------------------------------------------------------------------------------------
 typedef const __attribute__((address_space(1))) void* global_cptr;
 typedef __attribute__((address_space(3))) void* lds_ptr;
@@ -264,7 +265,16 @@ struct Gemm16 {
             if (uint32_t(st) < t.k_tiles) issue_slice(t, smem, st);
     }
 
+    // `after_first_barrier()` is called by every thread once, right behind the workgroup barrier that
+    // follows the wait for the tile's first slice. Every vector-memory operation a wavefront issued
+    // before begin() of this tile has completed by then, in every wavefront: what a persistent
+    // workgroup stored in the epilogue of its previous tile may be announced to other workgroups from
+    // there without a wait of its own. (begin() must follow the previous tile's finish().)
     static __device__ __forceinline__ void mainloop(const Tile& t, Acc& acc, char* smem) {
+        mainloop(t, acc, smem, [] {});
+    }
+    template <typename Hook>
+    static __device__ __forceinline__ void mainloop(const Tile& t, Acc& acc, char* smem, Hook&& after_first_barrier) {
         const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
         const int wm = wave / WAVES_N, wn = wave % WAVES_N;
         const int fr_row = lane & 31, fr_half = lane >> 5;
@@ -308,6 +318,7 @@ struct Gemm16 {
                 if (kt + 1 < t.k_tiles) wait_vmcnt<kLoadsPerSlice>();
                 else wait_vmcnt<0>();
                 asm volatile("s_barrier" ::: "memory");   // every wavefront's share of slice kt is in LDS
+                if (kt == 0) after_first_barrier();
                 const char* st = smem + stage_of(t, kt) * kStage;
                 read_fragments(st, 0);
 #pragma unroll
@@ -334,6 +345,7 @@ struct Gemm16 {
                 // every wavefront's share of slice kt is in LDS, and everyone has finished with the stage
                 // the next loads overwrite (slice kt-1, or the previous tile's epilogue staging)
                 asm volatile("s_barrier" ::: "memory");
+                if (kt == 0) after_first_barrier();
                 const char* st = smem + stage_of(t, kt) * kStage;
                 read_fragments(st, 0);
 #pragma unroll

@@ -12,8 +12,10 @@
 //     releases the down-projection tiles once all up-projection tiles of that block are stored
 //     (the reference's tQS counter + notifyNext, os/processor/processor.cuh:516-636,719-729).
 //     When the queues hold equal work the same tile list is walked without tickets: each XCD's
-//     workgroups stride through it by a rank they take at the start, with one barrier among them
-//     between the projections (the static schedule, chosen per launch inside the kernel).
+//     workgroups stride through it by a rank they take at the start (the static schedule, chosen
+//     per launch inside the kernel); the readiness counters stay, and since a queue lists all its
+//     up-projection tiles before its down-projection tiles they are normally complete long before
+//     they are looked at.
 #include "kernels.hpp"
 
 #include <type_traits>
@@ -91,12 +93,10 @@ __device__ __forceinline__ uint32_t kept_rows(const LayerParams& p, uint32_t e) 
 //   kSchedMembers + 32 (8 h + x)  workgroups of this launch that run on XCD x; h = launch parity
 //   kSchedReady + e*mt_max + m    readiness: up-projection tiles stored per (expert, row block)
 //   kSchedError                   set to non-zero by a workgroup whose bounded wait expired
-//   kSchedStaticRuns              launches so far that took the static schedule (they hold one more
-//                                 grid barrier, whose arrival counters advance only with them)
 constexpr uint32_t kSchedLine = 32;
-constexpr uint32_t kSchedBar = 0, kSchedError = 4, kSchedStaticRuns = 5, kSchedTicket = 4 * kSchedLine,
+constexpr uint32_t kSchedBar = 0, kSchedError = 4, kSchedTicket = 4 * kSchedLine,
                    kSchedGroup = 12 * kSchedLine, kSchedMembers = 44 * kSchedLine, kSchedReady = 60 * kSchedLine;
-constexpr uint32_t kGridBarriers = 4;
+constexpr uint32_t kGridBarriers = 3;
 // schedule of the expert phase of the persistent kernel (the values of kleos_amd.h's KLEOS_SCHEDULE_*)
 constexpr uint32_t kScheduleAuto = 0, kScheduleStatic = 2;   // anything else: dynamic
 static_assert(kSchedBar + kGridBarriers * kSchedLine <= kSchedTicket, "barrier words");
@@ -200,23 +200,6 @@ __device__ __forceinline__ uint32_t routed_count(const LayerParams& p, uint32_t 
     return total;
 }
 
-// Barrier among the `members` workgroups that run on XCD `xcd`, the `runs`-th time it is held on this
-// arena (counted from 0). The static schedule holds it between the two projections: a down tile
-// reads h1 rows that only workgroups of its own XCD stored.
-__device__ __forceinline__ void xcd_barrier(uint32_t* sched, unsigned long long ticks, uint32_t xcd, uint32_t runs, uint32_t members) {
-    wait_vmcnt<0>();   // the h1 stores of every wavefront, before the leader's release
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        uint32_t* arrived = sched + kSchedGroup + ((kGridBarriers - 1) * kXcds + xcd) * kSchedLine;
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-        atomic_add_agent(arrived, 1u);
-        const uint32_t target = (runs + 1u) * members;
-        bounded_wait(sched, ticks, [&] { return int32_t(atomic_load_relaxed(arrived) - target) >= 0; });
-    }
-    __syncthreads();
-    asm volatile("buffer_inv sc0" ::: "memory");   // drop this CU's L1; the rows are current in the XCD's L2
-}
-
 __device__ __forceinline__ bool balanced_or_forced(uint32_t policy, bool balanced) {
     return policy == kScheduleStatic || (policy == kScheduleAuto && balanced);
 }
@@ -231,7 +214,6 @@ struct Task {
     uint32_t dep;       // down tile: the readiness counter of its row block as seen when handed out
     uint32_t ready;     // down tile whose up-projection row block was already complete when handed out
     uint32_t valid;
-    uint32_t sync;      // not a tile (valid == 0): hold the grid barrier of the static schedule, then ask again
 };
 constexpr int kTaskWords = 12;
 
@@ -241,13 +223,13 @@ __device__ __forceinline__ Task broadcast_task(uint32_t* s_task, const Task& min
     if (threadIdx.x == 0) {
         s_task[0] = mine.e; s_task[1] = mine.kind; s_task[2] = mine.mtile; s_task[3] = mine.ntile;
         s_task[4] = mine.foreign; s_task[5] = mine.ready; s_task[6] = mine.valid; s_task[7] = mine.rows;
-        s_task[8] = mine.dep; s_task[9] = mine.sync;
+        s_task[8] = mine.dep;
     }
     __syncthreads();
     Task t;
     t.e = s_task[0]; t.kind = s_task[1]; t.mtile = s_task[2]; t.ntile = s_task[3];
     t.foreign = s_task[4]; t.ready = s_task[5]; t.valid = s_task[6]; t.rows = s_task[7];
-    t.dep = s_task[8]; t.sync = s_task[9];
+    t.dep = s_task[8];
     return t;
 }
 
@@ -297,6 +279,10 @@ struct Readiness {
     uint32_t* sched;      // nullptr: no cross-tile dependencies inside this launch (phased mode)
     uint32_t mt_max, tn_up;
     unsigned long long ticks;   // bound of a wait for a row block
+    // Every tile of a queue runs on the queue's own XCD (static schedule): a finished tile is in that
+    // XCD's L2 as soon as its stores are acknowledged, and its readers sit behind the same L2, so
+    // announcing it needs no write-back of the L2. With stealing a reader may sit anywhere.
+    bool local_only;
     __device__ __forceinline__ uint32_t* counter(const Task& t) const { return sched + kSchedReady + t.e * mt_max + t.mtile; }
     // A counter holds the stored tiles of the row block in its low half and, in its high half, how
     // many of them were stored by a workgroup on a foreign XCD (from whose L2 they were written back
@@ -312,11 +298,9 @@ struct Readiness {
 // `stats` (thread 0 only, may be null) accumulates 100 MHz ticks spent [0] fetching tasks,
 // [1] waiting for a dependency, [2] publishing, and counts [3] tiles, [4] tiles handed out before
 // their inputs were complete, [5] tiles taken from a foreign queue.
-// `mid_sync()` is called by every thread when `next` hands out a sync marker (static schedule
-// only: once per workgroup, between its last up tile and its first down tile).
-template <typename T, int V, typename Next, typename Sync>
+template <typename T, int V, typename Next>
 __device__ __forceinline__ void expert_loop(const LayerParams& p, char* smem, uint32_t* s_task, const Readiness rd,
-                                            unsigned long long* stats, Next&& next_raw, Sync&& mid_sync) {
+                                            unsigned long long* stats, Next&& next_raw) {
     const uint32_t tid = threadIdx.x;
     unsigned long long st_next = 0, st_wait = 0, st_pub = 0, n_tiles = 0, n_late = 0, n_foreign = 0;
     auto next = [&]() {
@@ -353,11 +337,11 @@ __device__ __forceinline__ void expert_loop(const LayerParams& p, char* smem, ui
         else asm volatile("buffer_inv sc0" ::: "memory");
     };
     auto publish = [&](const Task& t) {
-        // all stores of the tile are complete in every wavefront; make them visible device-wide,
-        // then count the tile (the reference's tQS increment, processor.cuh:719)
+        // all stores of the tile are complete in every wavefront; make them visible to whoever may
+        // read them, then count the tile (the reference's tQS increment, processor.cuh:719)
         if (rd.sched && t.kind == 0 && tid == 0) {
             const unsigned long long t0 = wall_clock64();
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+            if (!rd.local_only || t.foreign) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
             atomic_add_agent(rd.counter(t), t.foreign ? 1u + Readiness::kForeignUnit : 1u);
             st_pub += wall_clock64() - t0;
         }
@@ -376,47 +360,47 @@ __device__ __forceinline__ void expert_loop(const LayerParams& p, char* smem, ui
             g.act = o.act;
             return g;
         };
-        typename G::Tile cur_t, nxt_t;
+        typename G::Tile cur_t;
         typename G::Acc acc;
         Task cur = next();
-        if (cur.sync) { mid_sync(); cur = next(); }
         if (!cur.valid) { flush_stats(); return; }
         if (cur.kind == 1 && !cur.ready) wait_ready(cur);
         acquire(cur);
         int bias_slot = 0;
         G::begin(cur_t, args_of(cur), 0, bias_slot, smem);
-        for (;;) {
-            G::mainloop(cur_t, acc, smem);
-            Task nxt = next();   // its barrier: every wavefront has left the main loop
-            const bool early = nxt.valid && (nxt.kind == 0 || nxt.ready);
-            if (early) {
-                // the next tile's index look-ups and first loads travel while this tile's epilogue runs
-                acquire(nxt);
-                G::begin(nxt_t, args_of(nxt), G::next_stage0(cur_t), bias_slot ^= 1, smem);
-            }
-            G::finish(cur_t, acc, smem);
-            if (rd.sched && cur.kind == 0) {
-                // an up-projection tile other workgroups wait for: its stores must be complete in
-                // every wavefront before it is counted
+        // An up-projection tile whose stores are issued but which other workgroups have not been told
+        // of yet (valid == 0: none). Its stores are known to be complete behind the first barrier of
+        // the next tile's main loop, so it is counted from there, at no cost; it is counted at once,
+        // behind a wait for the stores, when the workgroup is about to block or to leave.
+        Task pending{};
+        auto publish_now = [&]() {
+            if (pending.valid) {
                 wait_vmcnt<0>();
                 __syncthreads();
-                publish(cur);
+                publish(pending);
+                pending.valid = 0;
             }
-            if (nxt.sync) { mid_sync(); nxt = next(); }
+        };
+        for (;;) {
+            G::mainloop(cur_t, acc, smem, [&] { if (pending.valid) publish(pending); });
+            pending.valid = 0;
+            const Task nxt = next();   // its barrier: every wavefront has left the main loop
+            G::finish(cur_t, acc, smem);
+            if (rd.sched && cur.kind == 0) pending = cur;
             if (!nxt.valid) break;
-            if (!early) {
-                if (nxt.kind == 1 && !nxt.ready) wait_ready(nxt);
-                acquire(nxt);
-                G::begin(nxt_t, args_of(nxt), G::next_stage0(cur_t), bias_slot ^= 1, smem);
-            }
             cur = nxt;
-            cur_t = nxt_t;
+            if (cur.kind == 1 && !cur.ready) {
+                publish_now();   // never wait while holding back a result of our own
+                wait_ready(cur);
+            }
+            acquire(cur);
+            G::begin(cur_t, args_of(cur), G::next_stage0(cur_t), bias_slot ^= 1, smem);
         }
+        publish_now();
         flush_stats();
     } else {
         for (;;) {
             Task t = next();
-            if (t.sync) { mid_sync(); continue; }
             if (!t.valid) break;
             if (t.kind == 1 && !t.ready) wait_ready(t);
             acquire(t);
@@ -489,7 +473,7 @@ __global__ __launch_bounds__((TileShape<T, V>::kThreads), (TileShape<T, V>::kPer
         }
         return broadcast_task(s_task, t);
     };
-    expert_loop<T, V>(p, gemm_smem + kPhasedGemmHeader, s_task, Readiness{nullptr, 0, 0, 0}, nullptr, next, [] {});
+    expert_loop<T, V>(p, gemm_smem + kPhasedGemmHeader, s_task, Readiness{nullptr, 0, 0, 0, true}, nullptr, next);
 }
 
 template <typename T>
@@ -520,11 +504,8 @@ __global__ __launch_bounds__((TileShape<T, V>::kThreads), (TileShape<T, V>::kPer
     // among the workgroups of its XCD, which the static schedule strides by.
     const uint32_t xcd = __builtin_amdgcn_s_getreg((3 << 11) | 20) & (kXcds - 1);
     uint32_t* const members_now = sched + kSchedMembers + (seq & 1u) * kXcds * kSchedLine;
-    uint32_t my_rank = 0, static_runs = 0;
-    if (tid == 0) {
-        my_rank = atomic_add_agent(members_now + xcd * kSchedLine, 1u);
-        static_runs = atomic_load_relaxed(sched + kSchedStaticRuns);
-    }
+    uint32_t my_rank = 0;
+    if (tid == 0) my_rank = atomic_add_agent(members_now + xcd * kSchedLine, 1u);
 
     // ---- phase 0: gate. Workgroup 0 also resets this launch's tickets and readiness counters
     // (nothing reads them before the second barrier) and the next launch's member counts.
@@ -561,10 +542,9 @@ __global__ __launch_bounds__((TileShape<T, V>::kThreads), (TileShape<T, V>::kPer
     uint32_t* s_qtot = s_qseg + 16;                                             // [8] tickets in each queue
     uint32_t* s_task = s_qtot + 8;                                              // [kTaskWords] task broadcast slot
     uint32_t* s_qup = s_task + kTaskWords;                                      // [8] up-projection tickets in each queue
-    // static schedule: [1] rank of the workgroup among those of its XCD,
-    // [2] static launches before this one, [3] next ticket of the workgroup, [4] the barrier between
-    // the projections is behind, [5] every XCD holds the same number of workgroups. Thread 0's own words live here rather than in registers that would
-    // stay occupied through the GEMM main loop.
+    // static schedule: [1] rank of the workgroup among those of its XCD, [3] next ticket of the
+    // workgroup, [5] every XCD holds the same number of workgroups. Thread 0's own words live here
+    // rather than in registers that would stay occupied through the GEMM main loop.
     uint32_t* s_static = s_qup + 8;
     static_assert((16 + 8 + kTaskWords + 8 + 6) * 4 <= kLdsQueue, "queue header");
     Segment* s_seg = reinterpret_cast<Segment*>(smem + lds_queue_offset(p.E) + kLdsQueue);   // at most 2*E segments
@@ -591,10 +571,10 @@ __global__ __launch_bounds__((TileShape<T, V>::kThreads), (TileShape<T, V>::kPer
         }
         __syncthreads();
         // Static or dynamic schedule: every workgroup decides alike, from the same counters.
-        // Static: each XCD's workgroups stride through their queue's up tiles, meet at a barrier, then
-        // stride through its down tiles: no tickets, no readiness counters, no per-tile publication.
-        // It needs every XCD to hold the same number of workgroups, and it pays only when no queue
-        // would keep its XCD busy for longer than freely handed-out tiles keep the grid busy.
+        // Static: each XCD's workgroups stride through their queue (all its up tiles, then all its
+        // down tiles) by their rank: no tickets, no stealing, nothing written back from the L2 per
+        // tile. It needs every XCD to hold the same number of workgroups, and it pays only when no
+        // queue would keep its XCD busy for longer than freely handed-out tiles keep the grid busy.
         // Thread q sets up queue q; its segments start at a fixed place, two per expert of the queue.
         const uint32_t my_nq = tid < p.E && tid < uint32_t(kXcds) ? (p.E - tid + kXcds - 1) / kXcds : 0u;   // experts q, q+8, ...
         if (tid < uint32_t(kXcds)) {
@@ -606,9 +586,7 @@ __global__ __launch_bounds__((TileShape<T, V>::kThreads), (TileShape<T, V>::kPer
             bool even = nwg % kXcds == 0;
             for (uint32_t j = 0; j < kXcds; ++j) even = even && seen[j] == members;
             s_static[1] = my_rank;
-            s_static[2] = static_runs;
             s_static[3] = my_rank;
-            s_static[4] = 0u;
             s_static[5] = even;
         }
         __syncthreads();
@@ -663,7 +641,7 @@ __global__ __launch_bounds__((TileShape<T, V>::kThreads), (TileShape<T, V>::kPer
     uint32_t q_off = 0;   // queues already found empty, starting from this workgroup's own XCD
     uint32_t q_dead = 0;  // bit q: queue q was seen exhausted
     bool q_scanned = false;
-    const Readiness rd{use_static ? nullptr : sched, mt_max, tn_up, p.wait_ticks};
+    const Readiness rd{sched, mt_max, tn_up, p.wait_ticks, use_static};
     auto decode = [&](Task& t, uint32_t q, uint32_t ticket) {
         uint32_t sg = s_qseg[q];
         const uint32_t sg_end = s_qseg[q + 1];
@@ -680,14 +658,10 @@ __global__ __launch_bounds__((TileShape<T, V>::kThreads), (TileShape<T, V>::kPer
         Task t{};
         if (tid == 0 && use_static) {
             const uint32_t ticket = s_static[3];
-            const bool down = s_static[4] != 0;
-            if (!down && ticket >= s_qup[xcd]) {
-                s_static[4] = 1u;
-                s_static[3] = s_qup[xcd] + s_static[1];
-                t.sync = 1;
-            } else if (ticket < (down ? s_qtot[xcd] : s_qup[xcd])) {
+            if (ticket < s_qtot[xcd]) {
                 decode(t, xcd, ticket);
-                t.ready = 1;
+                t.dep = t.kind == 0 ? 0u : atomic_load_relaxed(rd.counter(t));
+                t.ready = t.kind == 0 || rd.complete(t.dep);
                 s_static[3] = ticket + members;
             }
         } else if (tid == 0) {
@@ -714,12 +688,10 @@ __global__ __launch_bounds__((TileShape<T, V>::kThreads), (TileShape<T, V>::kPer
         }
         return broadcast_task(s_task, t);
     };
-    expert_loop<T, V>(p, s_gemm, s_task, rd, stamp + 8, next, [&] { xcd_barrier(sched, p.wait_ticks, xcd, s_static[2], members); });
+    expert_loop<T, V>(p, s_gemm, s_task, rd, stamp + 8, next);
     if (tid == 0) stamp[5] = wall_clock64();
     grid_barrier(sched, p.wait_ticks, 2, seq, nwg);
     if (tid == 0) stamp[6] = wall_clock64();
-    // every workgroup read the count when it started, before the first barrier
-    if (use_static && blockIdx.x == 0 && tid == 0) atomic_store_relaxed(sched + kSchedStaticRuns, s_static[2] + 1u);
 
     // ---- phase 3: combine, one token per wavefront
     if (p.is_training && blockIdx.x == nwg - 1 && wave == kWaves - 1) gate_loss_finalize(p);

@@ -170,10 +170,11 @@ int kleos_get_mode(void);
 
 /* How the persistent launch hands out expert tiles. The reference's scheduler is dynamic only
  * (csrc/include/kleos/os/scheduler.cuh); here the dynamic schedule (per-XCD ticket queues, readiness
- * counters, work stealing) has a static sibling: each XCD's workgroups stride through the
- * up-projection tiles of their queue, the grid meets at a barrier, and they stride through the
- * down-projection tiles. It spends nothing per tile on tickets and publication, and loses when the
- * queues hold unequal work. KLEOS_SCHEDULE_AUTO (default) decides inside the kernel, from the
+ * counters, work stealing) has a static sibling: each XCD's workgroups stride through their queue
+ * (all its up-projection tiles, then all its down-projection tiles) by a rank they take at the
+ * start; a down-projection tile still checks the readiness counter of its row block, which is
+ * normally complete long before. It spends nothing per tile on tickets or on writing results back
+ * from the L2 for readers on other XCDs, and loses when the queues hold unequal work. KLEOS_SCHEDULE_AUTO (default) decides inside the kernel, from the
  * routed counts of the launch: static when no XCD's queue takes its workgroups more rounds of tiles
  * than the whole tile list would take spread over all workgroups.
  * KLEOS_SCHEDULE_STATIC still falls back to the dynamic schedule when the hardware did not place
