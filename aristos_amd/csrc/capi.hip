@@ -52,11 +52,11 @@ size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 struct ArenaLayout {
     size_t logits, topk_expert, topk_prob, combine_den, topk_slot, tile_count, super_count,
-        expert_count, slot_token, h1, y, sched, stamps, tile_prob, super_prob, gate_loss, total;
+        expert_count, slot_token, h1, y, sched, stamps, tile_prob, super_prob, gate_loss, gate_partial, total;
     size_t zero_begin, zero_end;   // range that must start as zeros
 };
 
-ArenaLayout layout_arena(const kleos_config_t& c, uint32_t n_tiles, uint32_t n_super) {
+ArenaLayout layout_arena(const kleos_config_t& c, uint32_t n_tiles, uint32_t n_super, uint32_t gate_splits) {
     ArenaLayout L{};
     size_t off = 0;
     auto take = [&](size_t bytes) { size_t o = off; off = align_up(off + bytes, 256); return o; };
@@ -80,6 +80,7 @@ ArenaLayout layout_arena(const kleos_config_t& c, uint32_t n_tiles, uint32_t n_s
     L.slot_token = take(E * R * 4);
     L.h1 = take(E * R * size_t(c.I) * c.elem_bytes);
     L.y = take(E * R * size_t(c.H) * c.elem_bytes);
+    L.gate_partial = take(size_t(gate_splits) * S * c.PX * 4);
     L.total = off;
     return L;
 }
@@ -157,6 +158,7 @@ void params_from_arena(LayerParams& p, char* a, const ArenaLayout& L) {
     p.y = a + L.y;
     p.sched = reinterpret_cast<uint32_t*>(a + L.sched);
     p.stamps = reinterpret_cast<unsigned long long*>(a + L.stamps);
+    p.gate_partial = reinterpret_cast<float*>(a + L.gate_partial);
 }
 
 // Enqueues one forward. When ev is non-null (phased mode) it receives 6 recorded events that
@@ -173,7 +175,7 @@ int enqueue_forward(Context& c, const void* iP, void* oP, hipEvent_t* ev) {
         return KLEOS_OK;
     }
     if (ev) KLEOS_HIP(hipEventRecord(ev[0], c.stream));
-    KLEOS_HIP(launch_gate(p, dt, c.stream));
+    KLEOS_HIP(launch_gate(p, dt, c.num_cus, c.stream));
     if (ev) KLEOS_HIP(hipEventRecord(ev[1], c.stream));
     KLEOS_HIP(launch_slots(p, c.stream));
     if (ev) KLEOS_HIP(hipEventRecord(ev[2], c.stream));
@@ -249,7 +251,8 @@ extern "C" int kleos_moe_forward_static_scratch(const kleos_config_t* user_cfg, 
     if (!dev->gfx950) return fail(KLEOS_EUNSUPPORTED, "the current device is not gfx950: this library is built for MI355X only");
     LayerParams p{};
     params_from_config(p, cfg);
-    const ArenaLayout L = layout_arena(cfg, p.n_gate_tiles, p.n_super);
+    p.gate_splits = gate_splits_for(cfg.S, cfg.H, cfg.E, cfg.PX, int(cfg.torch_dtype), dev->num_cus);
+    const ArenaLayout L = layout_arena(cfg, p.n_gate_tiles, p.n_super, p.gate_splits);
     if (L.total > kStaticScratchBytes)
         return fail(KLEOS_EUNSUPPORTED, "kleos_moe_forward_static_scratch: this configuration needs %zu bytes of library "
                     "memory, the static scratch holds %zu; use kleos_initialize + kleos_moe_forward", L.total,
@@ -310,7 +313,11 @@ extern "C" int kleos_initialize_cfg(const kleos_config_t* user_cfg) {
 
     LayerParams& p = c->base;
     params_from_config(p, cfg);
-    const ArenaLayout L = layout_arena(cfg, p.n_gate_tiles, p.n_super);
+    p.gate_splits = gate_splits_for(cfg.S, cfg.H, cfg.E, cfg.PX, int(cfg.torch_dtype), c->num_cus);
+    if (size_t(p.gate_splits) * cfg.S * cfg.PX * 4 >= (size_t(1) << 31))
+        return bail(fail(KLEOS_EUNSUPPORTED, "the gate's partial sums (%u ranges x %u tokens x %u experts) exceed 2 GiB", p.gate_splits,
+                         cfg.S, cfg.PX));
+    const ArenaLayout L = layout_arena(cfg, p.n_gate_tiles, p.n_super, p.gate_splits);
     KLEOS_HIP_BAIL(hipMalloc(reinterpret_cast<void**>(&c->arena), L.total));
     c->arena_bytes = L.total;
     c->zero_begin = L.zero_begin;

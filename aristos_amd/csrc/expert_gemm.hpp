@@ -363,6 +363,37 @@ struct Gemm16 {
     // The stage the next tile's first slice must go to.
     static __device__ __forceinline__ int next_stage0(const Tile& t) { return (t.stage0 + t.k_tiles) % STAGES; }
 
+    // Epilogue that keeps the fp32 sums as they are (no bias, no activation, no rounding): the
+    // tile goes to out[m * ldo + n] as floats, for a caller that sums several K ranges of one product.
+    // Every wavefront must have left mainloop(). Each wavefront transposes its 32 x 32 blocks through
+    // 4 KB of its own in the stage of the last slice (rows of 128 bytes, chunk c of row r at position
+    // c ^ ((r >> 1) & 7)) and stores whole 128-byte lines.
+    static __device__ __forceinline__ void finish_partial(const Tile& t, Acc& acc, char* smem, float* out, uint32_t ldo) {
+        const uint32_t tid = local_tid();
+        const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+        const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+        const int fr_row = lane & 31, fr_half = lane >> 5;
+        char* stg = smem + last_stage(t) * kStage + wave * (kPanelRows * 128);
+#pragma unroll
+        for (int mi = 0; mi < TM; ++mi)
+#pragma unroll
+            for (int ni = 0; ni < TN; ++ni) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const f32x4 v{acc[ni][mi][4 * q], acc[ni][mi][4 * q + 1], acc[ni][mi][4 * q + 2], acc[ni][mi][4 * q + 3]};
+                    *reinterpret_cast<f32x4*>(stg + fr_row * 128 + (((2 * q + fr_half) ^ ((fr_row >> 1) & 7)) << 4)) = v;
+                }
+#pragma unroll
+                for (int it = 0; it < kPanelRows * 8 / kWave; ++it) {
+                    const int id = it * kWave + lane;
+                    const int r = id >> 3, c = id & 7;
+                    const u32x4 v = load16(stg + r * 128 + ((c ^ ((r >> 1) & 7)) << 4));
+                    const uint32_t m = wm * WM + mi * 32 + r, n = wn * WN + ni * 32 + c * 4;
+                    if (m < t.m_valid && n < t.n_valid) store16(out + size_t(m) * ldo + n, v);
+                }
+            }
+    }
+
     // Epilogue. Every wavefront must have left mainloop().
     static __device__ __forceinline__ void finish(const Tile& t, Acc& acc, char* smem) {
         const TileOut out{t.c_base, t.ldc, t.m_valid, t.n_valid, t.act};

@@ -289,6 +289,9 @@ __device__ __forceinline__ void gate_unit(const LayerParams& p, uint32_t unit, f
     __syncthreads();
 }
 
+template <typename T>
+__device__ __forceinline__ void gate_wide_epilogue(const LayerParams& p, uint32_t tile, float* smem, int lane);
+
 // The gate for more than 256 experts: one 16-token block per unit, the experts in passes of 256.
 // Every pass is the K loop and the reduction of gate_unit with 16 groups; wavefront 0 stores the
 // pass's logits, and when all passes are done it reads them back for softmax and top-k (each lane
@@ -368,7 +371,21 @@ __device__ __forceinline__ void gate_unit_wide(const LayerParams& p, uint32_t un
         __syncthreads();
     }
 
-    if (wave == 0 && live) {
+    if (wave == 0 && live) gate_wide_epilogue<T>(p, tile, smem, lane);
+    __syncthreads();
+}
+
+// Softmax, top-k, outputs and the tile histogram of one 16-token tile whose logits are in memory
+// (p.logits), run by one wavefront; `smem` holds E + 16 k words private to it. A lane reads the
+// logits it (or the wavefront that runs this) stored itself, or ones stored before a grid-wide
+// barrier: device-coherent loads either way.
+template <typename T>
+__device__ __forceinline__ void gate_wide_epilogue(const LayerParams& p, uint32_t tile, float* smem, int lane) {
+    const int col = lane & 15, chunk = lane >> 4;
+    const uint32_t E = p.E, k = p.k;
+    const uint32_t token = tile * kGateTileTokens + col;
+    float* my_logits = p.logits + size_t(token) * E;
+    {
         // lane (col, chunk) owns experts 16 j + 4 chunk + v of token col, as in the register gate
         const float kNegInf = -__builtin_inff();
         const uint32_t groups = (E + 15) / 16;
@@ -474,7 +491,65 @@ __device__ __forceinline__ void gate_unit_wide(const LayerParams& p, uint32_t un
             if (cnt) atomic_add_agent(super + e, cnt);
         }
     }
-    __syncthreads();
+}
+
+// ------------------------------------------------------------------------------------------------
+// Gate of the 16-bit Elements with more than 64 experts: the logits come from a tiled product
+// (128 tokens x 256 experts per workgroup, the hidden dimension split into p.gate_splits ranges
+// whose fp32 sums land in p.gate_partial[split][token][PX]), so the gate weights are read once per
+// 128 tokens instead of once per 16 or 32. After a grid-wide barrier one wavefront per 16-token
+// tile adds the ranges in ascending order (a fixed order: the logits do not depend on timing or on
+// the launch mode) and runs the same softmax / top-k / histogram code as the other gates.
+// ------------------------------------------------------------------------------------------------
+// The sum over the ranges of the 4 experts e0 .. e0+3 of `token` (e0 a multiple of 4; experts past
+// the padded count read as 0).
+__device__ __forceinline__ f32x4 gate_partial_sum(const LayerParams& p, coherent_rows_t partial, uint32_t token, uint32_t e0) {
+    f32x4 sum{0.f, 0.f, 0.f, 0.f};
+    if (e0 < p.PX) {
+        for (uint32_t s = 0; s < p.gate_splits; ++s) {
+            const uint32_t offset = ((s * p.S + token) * p.PX + e0) * 4u;
+            sum += __builtin_bit_cast(f32x4, load16_coherent(partial, offset));
+        }
+    }
+    return sum;
+}
+
+// Up to 256 experts: the sums go straight into the register layout of gate_epilogue.
+template <typename T, int NG>
+__device__ __forceinline__ void gate_reduce_tile(const LayerParams& p, uint32_t tile, int lane) {
+    const int col = lane & 15, chunk = lane >> 4;
+    const uint32_t token = tile * kGateTileTokens + col;
+    const coherent_rows_t partial = coherent_rows(p.gate_partial);
+    // range by range, the loads of all expert groups of a range in flight together; every sum runs
+    // over the ranges in ascending order
+    f32x4 acc[NG];
+#pragma unroll
+    for (int g = 0; g < NG; ++g) acc[g] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (uint32_t s = 0; s < p.gate_splits; ++s) {
+        const uint32_t row = ((s * p.S + token) * p.PX + 4 * chunk) * 4u;
+        u32x4 v[NG];
+#pragma unroll
+        for (int g = 0; g < NG; ++g) v[g] = uint32_t(16 * g + 4 * chunk) < p.PX ? load16_coherent(partial, row + 64u * g) : u32x4{0, 0, 0, 0};
+#pragma unroll
+        for (int g = 0; g < NG; ++g) acc[g] += __builtin_bit_cast(f32x4, v[g]);
+    }
+    gate_epilogue<T, NG>(p, tile, acc, lane);
+}
+
+// More than 256 experts: the sums go to p.logits, which the epilogue for many experts reads back.
+// `smem` holds E + 16 k words private to the calling wavefront.
+template <typename T>
+__device__ __forceinline__ void gate_reduce_tile_wide(const LayerParams& p, uint32_t tile, float* smem, int lane) {
+    const int col = lane & 15, chunk = lane >> 4;
+    const uint32_t token = tile * kGateTileTokens + col;
+    const coherent_rows_t partial = coherent_rows(p.gate_partial);
+    for (uint32_t e0 = 4 * chunk; e0 < p.E; e0 += 16) {
+        const f32x4 sum = gate_partial_sum(p, partial, token, e0);
+#pragma unroll
+        for (uint32_t v = 0; v < 4; ++v)
+            if (e0 + v < p.E) p.logits[size_t(token) * p.E + e0 + v] = sum[v];
+    }
+    gate_wide_epilogue<T>(p, tile, smem, lane);
 }
 
 // Slot assignment for one 16-token tile per wavefront. Every thread of the workgroup must call it

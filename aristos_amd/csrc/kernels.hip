@@ -96,7 +96,7 @@ __device__ __forceinline__ uint32_t kept_rows(const LayerParams& p, uint32_t e) 
 constexpr uint32_t kSchedLine = 32;
 constexpr uint32_t kSchedBar = 0, kSchedError = 4, kSchedTicket = 4 * kSchedLine,
                    kSchedGroup = 12 * kSchedLine, kSchedMembers = 44 * kSchedLine, kSchedReady = 60 * kSchedLine;
-constexpr uint32_t kGridBarriers = 3;
+constexpr uint32_t kGridBarriers = 4;   // 0 gate, 1 slots, 2 experts, 3 inside the gate (between its product and its epilogue)
 // schedule of the expert phase of the persistent kernel (the values of kleos_amd.h's KLEOS_SCHEDULE_*)
 constexpr uint32_t kScheduleAuto = 0, kScheduleStatic = 2;   // anything else: dynamic
 static_assert(kSchedBar + kGridBarriers * kSchedLine <= kSchedTicket, "barrier words");
@@ -416,7 +416,80 @@ __device__ __forceinline__ void expert_loop(const LayerParams& p, char* smem, ui
     }
 }
 
+// ------------------------------------------------------------------------------------ gate as a tiled product
+// Logits of the 16-bit Elements with more than 64 experts: tiles of 128 tokens x 256 experts over a
+// range of the hidden dimension, fp32 sums to p.gate_partial. Three stages of K slices (the gate
+// weights come from L2, the activations stream from HBM once).
+template <typename E>
+using GateGemm = Gemm16<E, 128, 256, 2, 4, 64, 3, false, false>;
+constexpr uint32_t kGateTileM = 128, kGateTileN = 256, kGateMaxSplits = 16;
+static_assert(GateGemm<bf16_t>::kThreads == kGemmThreads, "the gate product runs on the workgroups of the expert phase");
+
+__host__ __device__ inline uint32_t gate_gemm_tiles(const LayerParams& p) {
+    return (p.S / kGateTileM) * ceil_div_u32(p.PX, kGateTileN) * p.gate_splits;
+}
+
+// Tiles first, first + stride, ... of the gate product. Every thread of the workgroup must call it.
+template <typename T>
+__device__ __forceinline__ void gate_gemm_phase(const LayerParams& p, char* smem, uint32_t first, uint32_t stride) {
+    using G = GateGemm<T>;
+    const uint32_t tiles_n = ceil_div_u32(p.PX, kGateTileN), splits = p.gate_splits;
+    const uint32_t slices = p.H / uint32_t(G::kSliceK);
+    typename G::Tile t;
+    typename G::Acc acc;
+    for (uint32_t tile = first; tile < gate_gemm_tiles(p); tile += stride) {
+        // the ranges of one token block sit next to each other, so that they run at the same time
+        const uint32_t split = tile % splits, rest = tile / splits;
+        const uint32_t nb = rest % tiles_n, mb = rest / tiles_n;
+        const uint32_t k0 = (slices * split) / splits, k1 = (slices * (split + 1)) / splits;
+        GemmTileArgs g;
+        g.a_base = static_cast<const elem16_t*>(p.x) + size_t(mb) * kGateTileM * p.H + size_t(k0) * G::kSliceK;
+        g.a_row_index = nullptr; g.a_rows = p.S;
+        g.b_base = static_cast<const elem16_t*>(p.wg) + size_t(nb) * kGateTileN * p.H + size_t(k0) * G::kSliceK;
+        g.bias = static_cast<const elem16_t*>(p.wg);   // any readable 512 bytes: the sums take no bias
+        g.c_base = nullptr;
+        g.lda = p.H; g.ldb = p.H; g.ldc = 0; g.K = (k1 - k0) * G::kSliceK;
+        g.k_first = 0;
+        g.m_valid = kGateTileM;
+        g.n_valid = p.PX - nb * kGateTileN < kGateTileN ? p.PX - nb * kGateTileN : kGateTileN;
+        g.act = 2;
+        __syncthreads();   // every wavefront has left the previous tile's epilogue staging
+        if (k1 > k0) {
+            G::begin(t, g, 0, 0, smem);
+            G::mainloop(t, acc, smem);
+            __syncthreads();
+            float* out = p.gate_partial + (size_t(split) * p.S + size_t(mb) * kGateTileM) * p.PX + nb * kGateTileN;
+            G::finish_partial(t, acc, smem, out, p.PX);
+        }
+    }
+}
+
+// After the product: the 16-token tiles first, first + stride, ... of the calling wavefront.
+template <typename T, int NG>
+__device__ __forceinline__ void gate_reduce_phase(const LayerParams& p, float* wave_smem, uint32_t first, uint32_t stride) {
+    const int lane = threadIdx.x & 63;
+    for (uint32_t tile = first; tile < p.n_gate_tiles; tile += stride) {
+        if constexpr (NG == 0) gate_reduce_tile_wide<T>(p, tile, wave_smem, lane);
+        else gate_reduce_tile<T, NG>(p, tile, lane);
+    }
+}
+// LDS words per wavefront of the reduce phase (the many-expert epilogue keeps a histogram and the picks)
+__host__ __device__ inline uint32_t gate_reduce_wave_words(const LayerParams& p) { return p.E + kGateTileTokens * p.k; }
+
 // ------------------------------------------------------------------------------------ phased
+template <typename T>
+__global__ __launch_bounds__(kGemmThreads, 1) void gate_gemm_kernel(const LayerParams p) {
+    extern __shared__ __attribute__((aligned(16))) char gate_gemm_smem[];
+    if constexpr (sizeof(T) == 2) gate_gemm_phase<T>(p, gate_gemm_smem, blockIdx.x, gridDim.x);
+}
+template <typename T, int NG>
+__global__ __launch_bounds__(kPhaseThreads) void gate_reduce_kernel(const LayerParams p) {
+    extern __shared__ __attribute__((aligned(16))) float gate_reduce_smem[];
+    const uint32_t wave = threadIdx.x >> 6;
+    if constexpr (sizeof(T) == 2)
+        gate_reduce_phase<T, NG>(p, gate_reduce_smem + wave * gate_reduce_wave_words(p), blockIdx.x * 4 + wave, gridDim.x * 4);
+}
+
 // One gate unit per workgroup, with as many wavefronts as the persistent kernel's workgroups have:
 // the split of the hidden dimension, and with it the summation order of the logits, is the same
 // in both modes.
@@ -516,9 +589,22 @@ __global__ __launch_bounds__((TileShape<T, V>::kThreads), (TileShape<T, V>::kPer
         }
         for (uint32_t i = tid; i < p.E * mt_max; i += kThreads) sched[kSchedReady + i] = 0u;
     }
-    for (uint32_t unit = blockIdx.x; unit < ceil_div_u32(p.n_gate_tiles, gate_unit_blocks<NG>()); unit += nwg)
-        if constexpr (NG == 0) gate_unit_wide<T, int(kWaves)>(p, unit, reinterpret_cast<float*>(smem));
-        else gate_unit<T, NG, int(kWaves)>(p, unit, reinterpret_cast<float*>(smem));
+    bool gate_done = false;
+    if constexpr (sizeof(T) == 2 && (NG == 0 || NG >= 8)) {   // more than 64 experts
+        if (p.gate_splits) {
+            // logits as a tiled product, then (behind a grid-wide barrier) one wavefront per 16-token tile
+            gate_gemm_phase<T>(p, smem, blockIdx.x, nwg);
+            grid_barrier(sched, p.wait_ticks, 3, seq, nwg);
+            gate_reduce_phase<T, NG>(p, reinterpret_cast<float*>(smem) + wave * gate_reduce_wave_words(p), blockIdx.x + wave * nwg,
+                                     nwg * kWaves);
+            gate_done = true;
+        }
+    }
+    if (!gate_done)
+        for (uint32_t unit = blockIdx.x; unit < ceil_div_u32(p.n_gate_tiles, gate_unit_blocks<NG>()); unit += nwg) {
+            if constexpr (NG == 0) gate_unit_wide<T, int(kWaves)>(p, unit, reinterpret_cast<float*>(smem));
+            else gate_unit<T, NG, int(kWaves)>(p, unit, reinterpret_cast<float*>(smem));
+        }
     if (tid == 0) stamp[1] = wall_clock64();
     grid_barrier(sched, p.wait_ticks, 0, seq, nwg);
     if (tid == 0) stamp[2] = wall_clock64();
@@ -707,6 +793,12 @@ size_t fused_smem_bytes(uint32_t E) {
     const size_t slots = (TileShape<T>::kThreads / kWave) * size_t(E) * sizeof(uint32_t);
     if (gate > need) need = gate;
     if (slots > need) need = slots;
+    if constexpr (sizeof(T) == 2) {
+        const size_t product = GateGemm<T>::kSmemBytes;
+        const size_t reduce = (TileShape<T>::kThreads / kWave) * size_t(E + kGateTileTokens * kWideGateMaxK) * sizeof(float);
+        if (product > need) need = product;
+        if (reduce > need) need = reduce;
+    }
     return need;
 }
 
@@ -770,7 +862,47 @@ size_t sched_words(uint32_t E, uint32_t cap_rows) {
     return kSchedReady + size_t(E) * ceil_div_u32(cap_rows, 64) + 64;
 }
 
-hipError_t launch_gate(const LayerParams& p, int dtype, hipStream_t s) {
+uint32_t gate_splits_for(uint32_t S, uint32_t H, uint32_t E, uint32_t PX, int dtype, int num_cus) {
+    if ((dtype != 2 && dtype != 3) || E <= 64) return 0;
+    const uint32_t tiles = (S / kGateTileM) * ceil_div_u32(PX, kGateTileN);
+    uint32_t splits = ceil_div_u32(uint32_t(num_cus), tiles ? tiles : 1u);
+    const uint32_t slices = H / 64;
+    if (splits > slices) splits = slices;
+    if (splits > kGateMaxSplits) splits = kGateMaxSplits;
+    return splits < 1 ? 1u : splits;
+}
+
+hipError_t launch_gate(const LayerParams& p, int dtype, int num_cus, hipStream_t s) {
+    if (p.gate_splits) {
+        return dispatch_groups(p.E, [&](auto ng) {
+            constexpr int NG = decltype(ng)::value;
+            auto go = [&](auto tag) -> hipError_t {
+                using T = decltype(tag);
+                if constexpr (sizeof(T) == 2) {
+                    auto product = gate_gemm_kernel<T>;
+                    constexpr int smem = GateGemm<T>::kSmemBytes;
+                    static bool prepared = false;
+                    if (!prepared) {
+                        hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(product),
+                                                             hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+                        if (err != hipSuccess) return err;
+                        prepared = true;
+                    }
+                    uint32_t grid = gate_gemm_tiles(p);
+                    if (grid > uint32_t(num_cus)) grid = uint32_t(num_cus);
+                    hipLaunchKernelGGL(product, dim3(grid), dim3(kGemmThreads), smem, s, p);
+                    hipError_t err = hipGetLastError();
+                    if (err != hipSuccess) return err;
+                    hipLaunchKernelGGL((gate_reduce_kernel<T, NG>), dim3(ceil_div_u32(p.n_gate_tiles, 4)), dim3(kPhaseThreads),
+                                       4 * gate_reduce_wave_words(p) * sizeof(float), s, p);
+                    return hipGetLastError();
+                } else {
+                    return hipErrorInvalidValue;
+                }
+            };
+            return dispatch_dtype(dtype, go);
+        });
+    }
     return dispatch_groups(p.E, [&](auto ng) {
         constexpr int NG = decltype(ng)::value;
         auto go = [&](auto tag) -> hipError_t {

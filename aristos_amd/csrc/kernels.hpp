@@ -12,7 +12,11 @@ size_t sched_words(uint32_t E, uint32_t cap_rows);
 uint32_t sched_error_word();
 
 // Phase launchers (KLEOS_MODE_PHASED). dtype: 0 fp32, 2 bf16.
-hipError_t launch_gate(const LayerParams& p, int dtype, hipStream_t s);
+hipError_t launch_gate(const LayerParams& p, int dtype, int num_cus, hipStream_t s);
+// Ranges the gate splits the hidden dimension into when it computes its logits as a tiled product
+// (16-bit Elements, more than 64 experts); 0 when it does not. LayerParams::gate_partial then holds
+// splits * S * PX floats.
+uint32_t gate_splits_for(uint32_t S, uint32_t H, uint32_t E, uint32_t PX, int dtype, int num_cus);
 hipError_t launch_slots(const LayerParams& p, hipStream_t s);
 hipError_t launch_expert_gemm(const LayerParams& p, int dtype, int kind /*0 up, 1 down*/, int num_cus, hipStream_t s);
 hipError_t launch_combine(const LayerParams& p, int dtype, hipStream_t s);

@@ -34,6 +34,9 @@ struct LayerParams {
     uint32_t* super_count;    // [2][n_super, E]     the same summed over 32 tiles; two epochs
     uint32_t* expert_count;   // [E]
     int32_t* slot_token;      // [E, cap_rows]
+    // ---- gate logits as a tiled product (16-bit Elements, more than 64 experts)
+    float* gate_partial;      // [gate_splits][S, PX] fp32 sums over ranges of the hidden dimension
+    uint32_t gate_splits;     // 0: the gate computes its logits per 16-token tile, without this array
     // ---- training-mode gate loss (reference: gML / gMeC / gL, types.cuh:940-958)
     float* tile_prob;         // [n_gate_tiles, E]  sum of the tile's 16 probabilities of expert e
     float* super_prob;        // [n_super, E]       the same summed over 32 tiles
