@@ -61,6 +61,7 @@ SYMBOLS = {
     "kleos_get_mode": (C.c_int, []),
     "kleos_set_schedule": (C.c_int, [C.c_int]),
     "kleos_get_schedule": (C.c_int, []),
+    "kleos_set_cooperative_launch": (C.c_int, [C.c_int]),
     "kleos_schedule_taken": (C.c_int, [C.POINTER(C.c_int)]),
     "kleos_moe_debug_views": (C.c_int, [C.POINTER(DebugViewsStruct)]),
     "kleos_debug_copy_to_host": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t]),

@@ -392,6 +392,17 @@ extern "C" int kleos_set_schedule(int schedule) {
 
 extern "C" int kleos_get_schedule(void) { return g_ctx ? g_ctx->schedule : -1; }
 
+extern "C" int kleos_set_cooperative_launch(int on) {
+    if (int rc = require_ctx("kleos_set_cooperative_launch")) return rc;
+    if (on) {
+        int supported = 0;
+        KLEOS_HIP(hipDeviceGetAttribute(&supported, hipDeviceAttributeCooperativeLaunch, g_ctx->device));
+        if (!supported) return fail(KLEOS_EUNSUPPORTED, "kleos_set_cooperative_launch: the device does not support cooperative launches");
+    }
+    g_ctx->plan.cooperative = on != 0;
+    return KLEOS_OK;
+}
+
 extern "C" int kleos_schedule_taken(int* schedule) {
     if (int rc = require_ctx("kleos_schedule_taken")) return rc;
     if (!schedule) return fail(KLEOS_EINVAL, "kleos_schedule_taken: null argument");

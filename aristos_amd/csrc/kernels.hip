@@ -988,7 +988,8 @@ hipError_t plan_fused(const LayerParams& p, int dtype, int num_cus, FusedPlan* p
             if (err != hipSuccess) return err;
             if (occ < 1) return hipErrorLaunchOutOfResources;
             if (occ > 2) occ = 2;
-            // every workgroup must be resident at once: the kernel holds grid-wide barriers
+            // every workgroup must be resident at once: the kernel holds grid-wide barriers. The grid is
+            // what the occupancy query says fits an otherwise idle device.
             plan->nwg = uint32_t(num_cus) * uint32_t(occ);
             plan->smem = smem;
             const uint32_t cap = p.EC < p.cap_rows ? p.EC : p.cap_rows;
@@ -1012,6 +1013,9 @@ hipError_t launch_fused(const LayerParams& p, const FusedPlan& plan, uint32_t fu
     uint32_t mt_max = plan.mt_max, lag = plan.lag, policy = uint32_t(schedule);
     LayerParams pc = p;
     void* args[] = {&pc, &seq, &mt_max, &lag, &policy};
+    // A cooperative launch makes the runtime verify that the whole grid can be resident at once
+    // (it fails with hipErrorCooperativeLaunchTooLarge otherwise); it costs about 14 us per launch.
+    if (plan.cooperative) return hipLaunchCooperativeKernel(plan.kernel, dim3(plan.nwg), dim3(plan.threads), args, plan.smem, s);
     return hipLaunchKernel(plan.kernel, dim3(plan.nwg), dim3(plan.threads), args, plan.smem, s);
 }
 

@@ -30,6 +30,7 @@ struct FusedPlan {
     size_t smem = 0;
     uint32_t mt_max = 0;   // row blocks per expert at full capacity
     uint32_t lag = 0;      // experts between an up-projection segment and its down-projection segment
+    bool cooperative = false;   // launch through hipLaunchCooperativeKernel (residency verified per launch)
 };
 hipError_t plan_fused(const LayerParams& p, int dtype, int num_cus, FusedPlan* plan);
 // fused_seq: number of fused launches already issued on this scheduler arena.

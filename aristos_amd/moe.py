@@ -54,6 +54,12 @@ def set_schedule(schedule: int) -> None:
     _capi.check(_capi.lib().kleos_set_schedule(int(schedule)))
 
 
+def set_cooperative_launch(on: bool) -> None:
+    """Launch the persistent kernel through hipLaunchCooperativeKernel (the runtime then verifies per launch
+    that the whole grid is resident together; about 14 us more per launch)."""
+    _capi.check(_capi.lib().kleos_set_cooperative_launch(1 if on else 0))
+
+
 def schedule_taken() -> int:
     """SCHEDULE_DYNAMIC or SCHEDULE_STATIC: what the most recent persistent launch did."""
     out = C.c_int(-1)

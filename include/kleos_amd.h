@@ -182,6 +182,15 @@ int kleos_get_mode(void);
 enum { KLEOS_SCHEDULE_AUTO = 0, KLEOS_SCHEDULE_DYNAMIC = 1, KLEOS_SCHEDULE_STATIC = 2 };
 int kleos_set_schedule(int schedule);
 int kleos_get_schedule(void);
+/* The persistent kernel holds grid-wide barriers, so all its workgroups (one per compute unit) must
+ * be resident together. The library sizes the grid from the occupancy the runtime reports for an
+ * otherwise idle device; on a device that is busy with other kernels the barriers run into their
+ * time limit (see kleos_debug_set_wait_ticks) and the launch is reported as failed. With
+ * kleos_set_cooperative_launch(1) the kernel goes through hipLaunchCooperativeKernel instead, which
+ * makes the runtime itself check at every launch that the grid fits and return an error if it does not
+ * (measured: about 14 us more per launch, which is why it is off by default). The reference launches
+ * its persistent kernel plainly (moe.cuh:170, 198) and does not check. */
+int kleos_set_cooperative_launch(int on);
 /* The schedule the most recent persistent launch took: KLEOS_SCHEDULE_DYNAMIC or
  * KLEOS_SCHEDULE_STATIC. Synchronises the library stream. KLEOS_ESTATE before the first launch. */
 int kleos_schedule_taken(int* schedule);

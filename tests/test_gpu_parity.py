@@ -300,6 +300,30 @@ def test_timing_interfaces_of_the_persistent_launch():
     assert st["foreign_tiles"] <= st["tiles"]
 
 
+def test_cooperative_launch_gives_the_same_bits():
+    """kleos_set_cooperative_launch(1): the runtime checks the grid's residency at every launch; the
+    kernel and its results are the same."""
+    keys = _keys(1024, 256, 256, 16, 2)
+    c = moe_ref.cfg_from_keys(keys)
+    x, wg, w_up, w_down, *_ = random_layer(c, seed=10, w_std=0.06)
+    iP = _to_device(c, pack_inputs(c, x, wg, w_up, w_down))
+    _, plain, _ = run_gpu(keys, iP, ka.MODE_FUSED)
+    d = ka.initialize(keys)
+    try:
+        ka.moe.set_cooperative_launch(True)
+        oP = synth.alloc_outputs(d)
+        for _ in range(3):
+            ka.moe.forward_host(iP, oP)
+        ka.moe.stream_synchronize()
+        np.testing.assert_array_equal(_out_to_np(c, oP), _out_to_np(c, plain))
+        ka.moe.set_cooperative_launch(False)
+        ka.moe.forward_host(iP, oP)
+        ka.moe.stream_synchronize()
+        np.testing.assert_array_equal(_out_to_np(c, oP), _out_to_np(c, plain))
+    finally:
+        ka.finalize()
+
+
 def test_fused_and_phased_agree_bitwise():
     keys = _keys(1024, 256, 256, 16, 2)
     c = moe_ref.cfg_from_keys(keys)
