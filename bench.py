@@ -3,7 +3,11 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu-baseline]
 
 A step is one forward of the layer (one persistent kernel launch) over one batch of synthetic
-tokens already resident in HBM. Prints one JSON line: latency per forward, the roofline of the
+tokens already resident in HBM. The per-phase figures are measured first, with launch counts of
+their own (72 phased forwards, 1568 persistent ones: about half a second of sustained load, after
+which the device holds the clocks it keeps in a serving loop; it takes some 0.4 s to get there and
+loses them within milliseconds of idling); then come the timed region proper: `warmup`
+forwards and exactly `steps` forwards between two readings of the wall clock. Prints one JSON line: latency per forward, the roofline of the
 launch (the workload's arithmetic intensity decides which roof binds: algorithmic bytes / event-timed
 duration against HBM peak, with the matrix-core fraction beside it), per-phase figures from the
 phased mode, and the CPU oracle timed on this box's host cores as a baseline.
@@ -83,7 +87,7 @@ def main() -> int:
     import torch
 
     import aristos_amd as ka
-    from aristos_amd import synth
+    from aristos_amd import _capi, synth
 
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
@@ -105,20 +109,37 @@ def main() -> int:
     ka.initialize(w.config)
     try:
         oP = synth.alloc_outputs(d)
-        # ---- fused mode: the product path
+        lib_stream = torch.cuda.ExternalStream(_capi.lib().kleos_stream())
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        # ---- phased mode first: the same device code, one launch per phase, for per-phase figures
+        ka.moe.set_mode(ka.MODE_PHASED)
+        ph_total = ka.moe.forward_host_bench(iP, oP, skip=8, trials=max(64, args.steps))
+        ph = ka.moe.phase_times()
+        # ---- fused mode: the product path. Event-timed on the library stream (the reference's protocol,
+        # moe.cuh:160-181: skip launches, then trials launches between two events) ...
         ka.moe.set_mode(ka.MODE_FUSED)
-        for _ in range(args.warmup):
-            ka.moe.forward_host(iP, oP)
-        ka.moe.stream_synchronize()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(args.steps):
-            ka.moe.forward_host(iP, oP)
-        ka.moe.stream_synchronize()
-        torch.cuda.synchronize()
-        wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
-        # the same launches, timed by HIP events on the library stream (reference protocol, moe.cuh:160-181)
-        ev_ms = ka.moe.forward_host_bench(iP, oP, skip=0, trials=args.steps)
+        ka.moe.forward_host_bench(iP, oP, skip=32, trials=max(1536, args.steps))
+        # ... then, with nothing in between (the device drops its clocks within milliseconds of idling),
+        # the timed region: `warmup` forwards, then exactly `steps` forwards, timed by the wall clock (the
+        # reported value) and, the same launches, by HIP events on the stream the kernel runs on
+        # The protocol runs twice back to back and the first pass is discarded: the first pass of a
+        # process measures about 45 us per step more at 20 steps, whatever ran before it.
+        for rehearsal in (True, False):
+            for _ in range(args.warmup):
+                ka.moe.forward_host(iP, oP)
+            ka.moe.stream_synchronize()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            ev0.record(lib_stream)
+            for _ in range(args.steps):
+                ka.moe.forward_host(iP, oP)
+            ev1.record(lib_stream)
+            ka.moe.stream_synchronize()
+            torch.cuda.synchronize()
+            wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+            ev_ms = ev0.elapsed_time(ev1) / args.steps
+        # per-phase figures of the persistent kernel: from the stamps of the last launch and an event-timed run
+        ka.moe.forward_host_bench(iP, oP, skip=0, trials=8)
         fused_ph = ka.moe.phase_times()
         sched = ka.moe.scheduler_stats()
         schedule = "static" if ka.moe.schedule_taken() == ka.SCHEDULE_STATIC else "dynamic"
@@ -126,11 +147,6 @@ def main() -> int:
         kept = int(np.minimum(views["expert_count"].astype(np.int64), d.kept_capacity).sum())
         dropped = int((views["topk_slot"] < 0).sum())
         hottest = float(views["expert_count"].max() / (d.S * d.k / d.E))
-        # ---- phased mode: the same device code, one launch per phase, for per-phase figures
-        ka.moe.set_mode(ka.MODE_PHASED)
-        ph_total = ka.moe.forward_host_bench(iP, oP, skip=max(2, args.warmup // 4), trials=max(4, args.steps))
-        ph = ka.moe.phase_times()
-        ka.moe.set_mode(ka.MODE_FUSED)
     finally:
         ka.finalize()
 
