@@ -536,6 +536,167 @@ __device__ __forceinline__ void gate_reduce_tile(const LayerParams& p, uint32_t 
     gate_epilogue<T, NG>(p, tile, acc, lane);
 }
 
+// Up to 256 experts, a tile worked on by a group of four wavefronts (256 threads): wavefront w of
+// the group takes tokens 4 w .. 4 w + 3 of the tile, 16 lanes per token, each lane the experts
+// 64 j + 4 (lane % 16) + v (j < NL, NL * 64 >= PX, v < 4). Against one wavefront per tile every per-lane
+// loop over the experts is four times shorter, and the partial sums, logits and gate outputs move
+// in runs of 256 and 128 bytes per token. The tile's picks meet in LDS: one wavefront assigns the
+// in-tile ranks token by token (a token's k experts are distinct, so the lanes of a step never
+// touch the same histogram word), then the group writes the histogram out. Same sums over the
+// ranges, same selection rule and same order of the denominator as gate_epilogue; the softmax
+// denominator is summed in a different (fixed) order.
+// `gsm`: gate_group_words(p) words of LDS private to the group. Every thread of the workgroup must
+// call the function the same number of times (it contains workgroup barriers); a group without a
+// tile passes valid = false.
+__host__ __device__ inline uint32_t gate_group_words(uint32_t E, uint32_t k, bool training) {
+    return kGateTileTokens * k + E + (training ? kGateTileTokens * E : 0u);
+}
+template <typename T, int NL>
+__device__ __forceinline__ void gate_reduce_group(const LayerParams& p, uint32_t tile, bool valid, uint32_t* gsm, uint32_t gtid) {
+    constexpr uint32_t kGroupThreads = 4 * kWave;
+    const int lane = gtid & 63, sub = lane & 15;
+    const uint32_t gw = gtid >> 6, tl = 4 * gw + (lane >> 4);
+    const uint32_t E = p.E, k = p.k;
+    uint32_t* s_sel = gsm;                                   // [16][k] expert picked by token t in round r
+    uint32_t* s_hist = gsm + kGateTileTokens * k;            // [E]
+    float* s_prob = reinterpret_cast<float*>(s_hist + E);    // [16][E], training only
+    for (uint32_t e = gtid; e < E; e += kGroupThreads) s_hist[e] = 0u;
+    if (valid) {
+        const uint32_t token = tile * kGateTileTokens + tl;
+        const coherent_rows_t partial = coherent_rows(p.gate_partial);
+        f32x4 acc[NL];
+#pragma unroll
+        for (int j = 0; j < NL; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        // range by range, in ascending order; the loads of two ranges in flight together
+        for (uint32_t s0 = 0; s0 < p.gate_splits; s0 += 2) {
+            u32x4 v[2][NL];
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                const uint32_t s = s0 + u < p.gate_splits ? s0 + u : s0;
+                const uint32_t row = ((s * p.S + token) * p.PX + 4 * sub) * 4u;
+#pragma unroll
+                for (int j = 0; j < NL; ++j) v[u][j] = uint32_t(64 * j) < p.PX ? load16_coherent(partial, row + 256u * j) : u32x4{0, 0, 0, 0};
+            }
+#pragma unroll
+            for (int j = 0; j < NL; ++j) acc[j] += __builtin_bit_cast(f32x4, v[0][j]);
+            if (s0 + 1 < p.gate_splits) {
+#pragma unroll
+                for (int j = 0; j < NL; ++j) acc[j] += __builtin_bit_cast(f32x4, v[1][j]);
+            }
+        }
+        const float kNegInf = -__builtin_inff();
+        float m = kNegInf;
+#pragma unroll
+        for (int j = 0; j < NL; ++j)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const uint32_t e = 64 * j + 4 * sub + v;
+                if (e < E) p.logits[size_t(token) * E + e] = acc[j][v];
+                else acc[j][v] = kNegInf;   // softmax domain = the E real experts only (gate.cuh:550)
+                m = fmaxf(m, acc[j][v]);
+            }
+#pragma unroll
+        for (int off = 1; off <= 8; off <<= 1) m = fmaxf(m, __shfl_xor(m, off));
+        float d = 0.f;
+#pragma unroll
+        for (int j = 0; j < NL; ++j)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) d += __expf(acc[j][v] - m);
+#pragma unroll
+        for (int off = 1; off <= 8; off <<= 1) d += __shfl_xor(d, off);
+        const float inv_d = 1.0f / d;
+        auto prob = [&](float logit) { return __expf(logit - m) * inv_d; };
+        // gateOut[t, e] = Element(p) (gate.cuh:590-605); padded columns are zero
+        T* grow = static_cast<T*>(p.gate_out) + size_t(token) * p.PX;
+#pragma unroll
+        for (int j = 0; j < NL; ++j) {
+            T o[4];
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const uint32_t e = 64 * j + 4 * sub + v;
+                o[v] = float_to_elem<T>(e < E ? prob(acc[j][v]) : 0.f);
+                if (p.is_training && e < E) s_prob[tl * E + e] = prob(acc[j][v]);
+            }
+            static_assert(sizeof(T) == 2);
+            uint2 raw;
+            __builtin_memcpy(&raw, o, 8);
+            if (uint32_t(64 * j) < p.PX) *reinterpret_cast<uint2*>(grow + 64 * j + 4 * sub) = raw;
+        }
+        // top-k: k rounds of arg-max, equal values go to the lower expert index (gate.cuh:654-670);
+        // a picked expert leaves the working copy
+        f32x4 w[NL];
+#pragma unroll
+        for (int j = 0; j < NL; ++j) w[j] = acc[j];
+        float den = 0.f;
+        constexpr uint32_t kNone = 0x7fffffffu;
+        for (uint32_t r = 0; r < k; ++r) {
+            float best = kNegInf;
+            uint32_t bi = kNone;
+#pragma unroll
+            for (int j = 0; j < NL; ++j)
+#pragma unroll
+                for (int v = 0; v < 4; ++v)
+                    if (w[j][v] > best) {
+                        best = w[j][v];
+                        bi = 64 * j + 4 * sub + v;
+                    }
+#pragma unroll
+            for (int off = 1; off <= 8; off <<= 1) {
+                const float ob = __shfl_xor(best, off);
+                const uint32_t oi = __shfl_xor(bi, off);
+                if (oi != kNone && (bi == kNone || ob > best || (ob == best && oi < bi))) {
+                    best = ob;
+                    bi = oi;
+                }
+            }
+            // every lane of the token knows the winner and its logit
+            const float pv = bi != kNone ? prob(best) : 0.f;
+            den += pv;   // mCw, accumulated in selection order (gate.cuh:669)
+#pragma unroll
+            for (int j = 0; j < NL; ++j)
+#pragma unroll
+                for (int v = 0; v < 4; ++v)
+                    if (uint32_t(64 * j + 4 * sub + v) == bi) w[j][v] = kNegInf;
+            if (sub == 0) {
+                p.topk_expert[size_t(token) * k + r] = int32_t(bi);
+                p.topk_prob[size_t(token) * k + r] = pv;
+                s_sel[tl * k + r] = bi;
+            }
+        }
+        if (sub == 0) p.combine_den[token] = den;
+    }
+    __syncthreads();
+    // in-tile ranks (gate.cuh:678-696): token by token; LDS operations of one wavefront complete in order
+    if (valid && gw == 0) {
+        for (uint32_t t = 0; t < kGateTileTokens; ++t)
+            for (uint32_t r = lane; r < k; r += kWave) {
+                const uint32_t e = s_sel[t * k + r];
+                uint32_t rank = 0;
+                if (e < E) {
+                    rank = s_hist[e];
+                    s_hist[e] = rank + 1u;
+                }
+                p.topk_slot[(size_t(tile) * kGateTileTokens + t) * k + r] = int32_t(rank);
+            }
+    }
+    __syncthreads();
+    if (valid) {
+        uint32_t* super = p.super_count + size_t(p.epoch & 1u) * p.n_super * E + size_t(tile / kSuperTiles) * E;
+        for (uint32_t e = gtid; e < E; e += kGroupThreads) {
+            const uint32_t cnt = s_hist[e];
+            p.tile_count[size_t(tile) * E + e] = cnt;
+            if (cnt) atomic_add_agent(super + e, cnt);
+            if (p.is_training) {
+                // column sums of the tile's probabilities for the load-balancing loss (gate.cuh:608-635)
+                float col_sum = 0.f;
+                for (uint32_t t = 0; t < kGateTileTokens; ++t) col_sum += s_prob[t * E + e];
+                p.tile_prob[size_t(tile) * E + e] = col_sum;
+            }
+        }
+    }
+    __syncthreads();   // the next tile clears the histogram
+}
+
 // More than 256 experts: the sums go to p.logits, which the epilogue for many experts reads back.
 // `smem` holds E + 16 k words private to the calling wavefront.
 template <typename T>

@@ -464,17 +464,37 @@ __device__ __forceinline__ void gate_gemm_phase(const LayerParams& p, char* smem
     }
 }
 
-// After the product: the 16-token tiles first, first + stride, ... of the calling wavefront.
+__host__ __device__ inline uint32_t gate_reduce_wave_words(const LayerParams& p);
+// After the product: the 16-token tiles wg, wg + nwg, ... of the calling workgroup. Up to 256
+// experts a tile goes to a group of four wavefronts (gate_reduce_group), above to a single one.
+// Every thread of the workgroup must call it (workgroup barriers inside).
 template <typename T, int NG>
-__device__ __forceinline__ void gate_reduce_phase(const LayerParams& p, float* wave_smem, uint32_t first, uint32_t stride) {
-    const int lane = threadIdx.x & 63;
-    for (uint32_t tile = first; tile < p.n_gate_tiles; tile += stride) {
-        if constexpr (NG == 0) gate_reduce_tile_wide<T>(p, tile, wave_smem, lane);
-        else gate_reduce_tile<T, NG>(p, tile, lane);
+__device__ __forceinline__ void gate_reduce_phase(const LayerParams& p, float* smem, uint32_t wg, uint32_t nwg) {
+    const uint32_t tid = threadIdx.x, waves = blockDim.x / kWave;
+    if constexpr (NG == 0) {
+        const uint32_t wave = tid / kWave;
+        float* wave_smem = smem + wave * gate_reduce_wave_words(p);
+        for (uint32_t tile = wg + wave * nwg; tile < p.n_gate_tiles; tile += nwg * waves)   // spread over the workgroups first
+            gate_reduce_tile_wide<T>(p, tile, wave_smem, int(tid % kWave));
+    } else {
+        constexpr int NL = (NG + 3) / 4;   // runs of 64 experts
+        const uint32_t groups = waves / 4, group = tid / (4 * kWave), gtid = tid % (4 * kWave);
+        uint32_t* gsm = reinterpret_cast<uint32_t*>(smem) + group * gate_group_words(p.E, p.k, p.is_training != 0);
+        // tiles wg + j * nwg of the workgroup, j = 0 .. count-1; group g takes j = g, g + groups, ...
+        const uint32_t count = wg < p.n_gate_tiles ? ceil_div_u32(p.n_gate_tiles - wg, nwg) : 0u;
+        for (uint32_t j0 = 0; j0 < count; j0 += groups) {
+            const uint32_t j = j0 + group;
+            gate_reduce_group<T, NL>(p, wg + j * nwg, j < count, gsm, gtid);
+        }
     }
 }
-// LDS words per wavefront of the reduce phase (the many-expert epilogue keeps a histogram and the picks)
+// LDS words per wavefront of the reduce phase for more than 256 experts (a histogram and the picks)
 __host__ __device__ inline uint32_t gate_reduce_wave_words(const LayerParams& p) { return p.E + kGateTileTokens * p.k; }
+// LDS bytes of the reduce phase of a workgroup of `threads` threads
+inline size_t gate_reduce_smem_bytes(const LayerParams& p, uint32_t threads) {
+    if (p.E > 256) return size_t(threads / kWave) * gate_reduce_wave_words(p) * sizeof(float);
+    return size_t(threads / (4 * kWave)) * gate_group_words(p.E, p.k, p.is_training != 0) * sizeof(float);
+}
 
 // ------------------------------------------------------------------------------------ phased
 template <typename T>
@@ -485,9 +505,7 @@ __global__ __launch_bounds__(kGemmThreads, 1) void gate_gemm_kernel(const LayerP
 template <typename T, int NG>
 __global__ __launch_bounds__(kPhaseThreads) void gate_reduce_kernel(const LayerParams p) {
     extern __shared__ __attribute__((aligned(16))) float gate_reduce_smem[];
-    const uint32_t wave = threadIdx.x >> 6;
-    if constexpr (sizeof(T) == 2)
-        gate_reduce_phase<T, NG>(p, gate_reduce_smem + wave * gate_reduce_wave_words(p), blockIdx.x * 4 + wave, gridDim.x * 4);
+    if constexpr (sizeof(T) == 2) gate_reduce_phase<T, NG>(p, gate_reduce_smem, blockIdx.x, gridDim.x);
 }
 
 // One gate unit per workgroup, with as many wavefronts as the persistent kernel's workgroups have:
@@ -595,8 +613,7 @@ __global__ __launch_bounds__((TileShape<T, V>::kThreads), (TileShape<T, V>::kPer
             // logits as a tiled product, then (behind a grid-wide barrier) one wavefront per 16-token tile
             gate_gemm_phase<T>(p, smem, blockIdx.x, nwg);
             grid_barrier(sched, p.wait_ticks, 3, seq, nwg);
-            gate_reduce_phase<T, NG>(p, reinterpret_cast<float*>(smem) + wave * gate_reduce_wave_words(p), blockIdx.x + wave * nwg,
-                                     nwg * kWaves);
+            gate_reduce_phase<T, NG>(p, reinterpret_cast<float*>(smem), blockIdx.x, nwg);
             gate_done = true;
         }
     }
@@ -795,7 +812,10 @@ size_t fused_smem_bytes(uint32_t E) {
     if (slots > need) need = slots;
     if constexpr (sizeof(T) == 2) {
         const size_t product = GateGemm<T>::kSmemBytes;
-        const size_t reduce = (TileShape<T>::kThreads / kWave) * size_t(E + kGateTileTokens * kWideGateMaxK) * sizeof(float);
+        // reduce phase: per wavefront a histogram and the picks (more than 256 experts), or per group
+        // of four wavefronts the picks, a histogram and the probabilities of a tile (k <= E <= 256)
+        const size_t reduce = E > 256 ? (TileShape<T>::kThreads / kWave) * size_t(E + kGateTileTokens * kWideGateMaxK) * sizeof(float)
+                                      : (TileShape<T>::kThreads / (4 * kWave)) * size_t(gate_group_words(256, 256, true)) * sizeof(float);
         if (product > need) need = product;
         if (reduce > need) need = reduce;
     }
@@ -893,8 +913,10 @@ hipError_t launch_gate(const LayerParams& p, int dtype, int num_cus, hipStream_t
                     hipLaunchKernelGGL(product, dim3(grid), dim3(kGemmThreads), smem, s, p);
                     hipError_t err = hipGetLastError();
                     if (err != hipSuccess) return err;
-                    hipLaunchKernelGGL((gate_reduce_kernel<T, NG>), dim3(ceil_div_u32(p.n_gate_tiles, 4)), dim3(kPhaseThreads),
-                                       4 * gate_reduce_wave_words(p) * sizeof(float), s, p);
+                    // one tile per group of four wavefronts (per wavefront above 256 experts)
+                    const uint32_t reduce_grid = p.E > 256 ? ceil_div_u32(p.n_gate_tiles, kPhaseThreads / kWave) : p.n_gate_tiles;
+                    hipLaunchKernelGGL((gate_reduce_kernel<T, NG>), dim3(reduce_grid), dim3(kPhaseThreads),
+                                       gate_reduce_smem_bytes(p, kPhaseThreads), s, p);
                     return hipGetLastError();
                 } else {
                     return hipErrorInvalidValue;

@@ -143,6 +143,8 @@ CASES = [
     (512, 128, 128, 64, 2, 1.0, 1, 0, 2, 0.0),     # E = 64
     (256, 128, 64, 130, 8, 1.0, 1, 0, 2, 0.0),     # E > 128 (gate handles up to 256 experts)
     (256, 128, 64, 256, 8, 1.0, 1, 0, 2, 0.0),     # E = 256, top-8
+    (128, 128, 64, 96, 72, 1.0, 1, 0, 3, 0.0),     # fp16, 64 < E <= 256 with k > 64: more picks per token than a wavefront has lanes
+    (256, 128, 64, 200, 5, 1.5, 1, 0, 3, 0.1),     # fp16, E = 200 (padded to 256 columns, not a multiple of 16)
     (256, 128, 192, 8, 2, 1.0, 1, 1, 0, 0.1),      # fp32 + gelu
     (256, 64, 64, 24, 3, 1.0, 1, 0, 0, 0.0),       # fp32, E = 24
     (1024, 192, 320, 4, 2, 1.0, 1, 0, 2, 0.1),     # 512 rows per expert: 256-row tiles, odd slice counts
