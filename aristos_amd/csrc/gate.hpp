@@ -497,9 +497,10 @@ __device__ __forceinline__ void gate_wide_epilogue(const LayerParams& p, uint32_
 // Gate of the 16-bit Elements with more than 64 experts: the logits come from a tiled product
 // (128 tokens x 256 experts per workgroup, the hidden dimension split into p.gate_splits ranges
 // whose fp32 sums land in p.gate_partial[split][token][PX]), so the gate weights are read once per
-// 128 tokens instead of once per 16 or 32. After a grid-wide barrier one wavefront per 16-token
-// tile adds the ranges in ascending order (a fixed order: the logits do not depend on timing or on
-// the launch mode) and runs the same softmax / top-k / histogram code as the other gates.
+// 128 tokens instead of once per 16 or 32. After a grid-wide barrier the 16-token tiles are
+// reduced - by a group of four wavefronts each up to 256 experts, by one wavefront above: the
+// ranges are added in ascending order (a fixed order: the logits do not depend on timing or on the
+// launch mode), then softmax, top-k and the tile's histogram as in the other gates.
 // ------------------------------------------------------------------------------------------------
 // The sum over the ranges of the 4 experts e0 .. e0+3 of `token` (e0 a multiple of 4; experts past
 // the padded count read as 0).
@@ -512,28 +513,6 @@ __device__ __forceinline__ f32x4 gate_partial_sum(const LayerParams& p, coherent
         }
     }
     return sum;
-}
-
-// Up to 256 experts: the sums go straight into the register layout of gate_epilogue.
-template <typename T, int NG>
-__device__ __forceinline__ void gate_reduce_tile(const LayerParams& p, uint32_t tile, int lane) {
-    const int col = lane & 15, chunk = lane >> 4;
-    const uint32_t token = tile * kGateTileTokens + col;
-    const coherent_rows_t partial = coherent_rows(p.gate_partial);
-    // range by range, the loads of all expert groups of a range in flight together; every sum runs
-    // over the ranges in ascending order
-    f32x4 acc[NG];
-#pragma unroll
-    for (int g = 0; g < NG; ++g) acc[g] = f32x4{0.f, 0.f, 0.f, 0.f};
-    for (uint32_t s = 0; s < p.gate_splits; ++s) {
-        const uint32_t row = ((s * p.S + token) * p.PX + 4 * chunk) * 4u;
-        u32x4 v[NG];
-#pragma unroll
-        for (int g = 0; g < NG; ++g) v[g] = uint32_t(16 * g + 4 * chunk) < p.PX ? load16_coherent(partial, row + 64u * g) : u32x4{0, 0, 0, 0};
-#pragma unroll
-        for (int g = 0; g < NG; ++g) acc[g] += __builtin_bit_cast(f32x4, v[g]);
-    }
-    gate_epilogue<T, NG>(p, tile, acc, lane);
 }
 
 // Up to 256 experts, a tile worked on by a group of four wavefronts (256 threads): wavefront w of

@@ -46,9 +46,11 @@ constexpr int kXcds = 8;
 // Variants 0 and 1 load their weight rows non-temporally (headline 378 against 390 us per forward,
 // the 16-expert shape 192 against 196, the 256-expert shape 3.43 against 3.48 ms); variant 2, whose
 // weight tiles are shared by eight workgroups and more, does not (4.06 against 4.01 ms with it).
+// Variant 1 also writes its output rows through the L2 (the 256-expert shape stores 0.58 GB per
+// launch: 3.03 against 3.11 ms per forward; no difference on the shapes of variants 0 and 2).
 template <typename E, int V>
 using GemmCfg = std::conditional_t<V == 0, Gemm16<E, 256, 256, 2, 4, 64, 2, true, true>,
-                std::conditional_t<V == 1, Gemm16<E, 128, 256, 2, 4, 64, 3, true, false>, Gemm16<E, 256, 256, 2, 4, 64, 2, false, false>>>;
+                std::conditional_t<V == 1, Gemm16<E, 128, 256, 2, 4, 64, 3, true, false, true>, Gemm16<E, 256, 256, 2, 4, 64, 2, false, false>>>;
 constexpr int kBN = 256;
 constexpr int kGemmThreads = GemmCfg<bf16_t, 0>::kThreads;
 static_assert(GemmCfg<bf16_t, 1>::kThreads == kGemmThreads && GemmCfg<bf16_t, 2>::kThreads == kGemmThreads,
