@@ -1,4 +1,4 @@
-// Weighted combine: out[t] = sum over the kept experts of t of  Element(p_e) * Element(y_e / den_t).
+// Weighted combine: out[t] = sum over the kept experts of t of  Element(p_e) * Element(y_e * (1 / den_t)).
 //
 // Replaces processor::combine (csrc/include/kleos/os/processor/processor.cuh:44-205). The
 // reference scatters each expert tile into the output with Element atomicAdd, in arrival order,
@@ -55,7 +55,9 @@ __device__ __forceinline__ void combine_tokens_inline(const LayerParams& p, uint
     for (uint32_t token = first; token < p.S; token += stride) {
         CombineRoute<KMAX> nxt = cur;
         if (token + stride < p.S) nxt = combine_route<KMAX>(p, token + stride);
-        const float den = cur.den;
+        // y / den as y * (1 / den): the reference divides with __fdividef (processor.cuh:135), an
+        // approximate division, and a full IEEE division per element made this phase instruction-bound
+        const float inv_den = __builtin_amdgcn_rcpf(cur.den);
         coherent_rows_t rows[KMAX];
         float scale[KMAX];
         bool on[KMAX];
@@ -80,7 +82,7 @@ __device__ __forceinline__ void combine_tokens_inline(const LayerParams& p, uint
 #pragma unroll
             for (int c = 0; c < CH; ++c) {
                 if (c0 + c * col_stride >= H) break;
-                // Element(gateOut[t, e]) * Element(fp32(y) / den), summed in fp32 in selection order
+                // Element(gateOut[t, e]) * Element(fp32(y) * (1 / den)), summed in fp32 in selection order
                 // (processor.cuh:117,135,146); with k == 1 the row is copied unscaled
                 // (processor.cuh:170-203).
                 float acc[kPer];
@@ -94,7 +96,7 @@ __device__ __forceinline__ void combine_tokens_inline(const LayerParams& p, uint
 #pragma unroll
                     for (int j = 0; j < kPer; ++j) {
                         if (k == 1) acc[j] = elem_to_float(vals[j]);
-                        else acc[j] = fmaf(scale[r], elem_to_float(float_to_elem<T>(elem_to_float(vals[j]) / den)), acc[j]);
+                        else acc[j] = fmaf(scale[r], elem_to_float(float_to_elem<T>(elem_to_float(vals[j]) * inv_den)), acc[j]);
                     }
                 }
                 T o[kPer];
@@ -117,7 +119,7 @@ __device__ __forceinline__ void combine_tokens_generic(const LayerParams& p, uin
     const uint32_t H = p.H, k = p.k;
     const T* y = static_cast<const T*>(p.y);
     for (uint32_t token = first; token < p.S; token += stride) {
-        const float den = load_coherent(p.combine_den + token);
+        const float inv_den = __builtin_amdgcn_rcpf(load_coherent(p.combine_den + token));
         T* out = static_cast<T*>(p.moe_out) + size_t(token) * H;
         for (uint32_t c0 = lane * kPer; c0 < H; c0 += kWave * kPer) {
             float acc[kPer];
@@ -134,7 +136,7 @@ __device__ __forceinline__ void combine_tokens_generic(const LayerParams& p, uin
                 __builtin_memcpy(vals, &raw, 16);
 #pragma unroll
                 for (int j = 0; j < kPer; ++j)
-                    acc[j] = fmaf(scale, elem_to_float(float_to_elem<T>(elem_to_float(vals[j]) / den)), acc[j]);
+                    acc[j] = fmaf(scale, elem_to_float(float_to_elem<T>(elem_to_float(vals[j]) * inv_den)), acc[j]);
             }
             T o[kPer];
 #pragma unroll
