@@ -305,7 +305,7 @@ __device__ __forceinline__ void gate_unit_wide(const LayerParams& p, uint32_t un
     constexpr int NG = 16;
     const int wave = __builtin_amdgcn_readfirstlane(int(threadIdx.x >> 6)), lane = threadIdx.x & 63;
     const int col = lane & 15, chunk = lane >> 4;
-    const uint32_t H = p.H, E = p.E, k = p.k;
+    const uint32_t H = p.H, E = p.E;
     constexpr int kStepK = GateK<T>::kStepK;
     constexpr int kPer = GateK<T>::kElemsPer16B;
     const uint32_t steps = H / kStepK;
