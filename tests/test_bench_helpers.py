@@ -1,0 +1,40 @@
+"""Host-side pieces of bench.py that need no GPU: the source fingerprint and the HBM traffic figure
+it reads out of the committed counter summaries."""
+import os
+import subprocess
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, ROOT)
+import bench  # noqa: E402
+
+WORKLOADS = ["headline_e64_zipf", "balanced_e16", "mixtral_e8", "fine_e256_top8"]
+
+
+def test_fingerprint_is_stable_and_covers_the_sources():
+    a, b = bench.source_fingerprint(), bench.source_fingerprint()
+    assert a == b and len(a) == 16 and int(a, 16) >= 0
+
+
+@pytest.mark.parametrize("workload", WORKLOADS)
+def test_committed_traffic_summary_is_readable(workload):
+    """Every profiled workload has a summary bench.py can read: a positive byte count that is at
+    least the weights once (nothing can stream less than that) and below ten times that."""
+    from aristos_amd import synth
+    d = synth.WORKLOADS[workload].config.derive()
+    nbytes, same_sources = bench.measured_traffic(workload)
+    assert nbytes is not None and same_sources in (True, False)
+    weights = 2.0 * d.E * d.H * d.I * d.elem_bytes
+    assert 0.95 * weights < nbytes < 10.0 * weights
+
+
+def test_unknown_workload_has_no_traffic_figure():
+    assert bench.measured_traffic("no_such_workload") == (None, None)
+
+
+def test_more_than_one_gpu_is_refused_with_a_message():
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert r.returncode != 0
+    assert "one GPU" in (r.stdout + r.stderr) or "1 GPU" in (r.stdout + r.stderr) or "single" in (r.stdout + r.stderr).lower()
