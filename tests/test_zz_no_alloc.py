@@ -105,3 +105,33 @@ def test_static_scratch_refuses_what_does_not_fit():
     msg = _capi.lib().kleos_last_error().decode()
     assert "static scratch holds 33554432" in msg, msg
     torch.cuda.synchronize()
+
+
+def test_static_scratch_forward_replays_from_a_graph():
+    """The entry point exists for callers under stream capture: recorded once into a HIP graph, every
+    replay gives the bits of kleos_moe_forward, with eager calls on the same array between the replays
+    (the counters are cleared by a fill kernel, which a graph replays faithfully)."""
+    keys = _keys(1024, 256, 512, 16, 2)
+    c, iP = _device_inputs(keys, 71)
+    d, ref = _existing_entry_point(keys, iP)
+    ref = _bits(c, ref)
+    oP = synth.alloc_outputs(d)
+    side = torch.cuda.Stream()
+    ka.moe.forward_static_scratch(keys, iP, oP, stream=side.cuda_stream)   # the per-device set-up happens eagerly
+    side.synchronize()
+    np.testing.assert_array_equal(_bits(c, oP), ref)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        ka.moe.forward_static_scratch(keys, iP, oP, stream=torch.cuda.current_stream().cuda_stream)
+    other = _keys(256, 128, 128, 8, 2, cf=2.0)
+    c2, iP2 = _device_inputs(other, 72)
+    oP2 = synth.alloc_outputs(other.derive())
+    for _ in range(4):
+        oP.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(_bits(c, oP), ref)
+        # eager work on the same array, of another shape, between the replays
+        ka.moe.forward_static_scratch(other, iP2, oP2)
+        torch.cuda.synchronize()
