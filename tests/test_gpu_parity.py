@@ -175,6 +175,27 @@ def test_shapes_and_edges(mode, S, H, I, E, k, cf, drop, act, dt, bias):
     check_against_oracle(c, keys, iP, mode)
 
 
+def _drawn_case(index):
+    """A configuration drawn from a fixed seed: sizes, expert count (1 to 512, around every boundary of
+    the gate variants), top-k, capacity factor, activation, Element type and bias at random."""
+    import random
+    rng = random.Random(1000 + index)
+    S = rng.choice([128, 256, 384, 512, 1024])
+    H, I = 64 * rng.randint(1, 8), 64 * rng.randint(1, 8)
+    E = rng.choice([1, 2, 3, 5, 8, 12, 16, 24, 33, 64, 65, 70, 96, 128, 129, 130, 192, 200, 255, 256, 257, 300, 384, 500, 512])
+    k = rng.randint(1, min(E, rng.choice([2, 4, 8, 16, 32])))
+    cf = rng.choice([1.0, 1.0, 1.25, 1.5, 2.5, 4.0])
+    return (S, H, I, E, k, cf, rng.choice([0, 1, 1]), rng.choice([0, 1]), rng.choice([2, 2, 3, 0]), rng.choice([0.0, 0.1]))
+
+
+@pytest.mark.parametrize("index", range(12))
+def test_drawn_configurations(index):
+    """Twelve configurations nobody picked by hand, each through the phased launches and the persistent
+    launch under both schedules."""
+    for mode in MODES:
+        test_shapes_and_edges(mode, *_drawn_case(index))
+
+
 @pytest.mark.parametrize("mode", MODES, ids=MODE_IDS)
 def test_exact_ties_go_to_the_lower_index(mode):
     """Duplicate gate rows give bit-identical logits for expert pairs; the lower index must win, and
