@@ -7,6 +7,7 @@
 // gemm.cuh:22-107). Rounding points are the reference's: fp32 accumulate, fp32 bias add and
 // activation, one round-to-nearest-even to Element on store (processor.cuh:475).
 #pragma once
+#include <type_traits>
 #include "device_common.hpp"
 
 namespace kleos_amd {
@@ -312,57 +313,91 @@ struct Gemm16 {
 #pragma unroll
             for (int mi = 0; mi < TM; ++mi) fx[ks & 1][mi] = __builtin_bit_cast(vec8, load16(st + (base_x ^ (ks << 5)) + mi * 32 * kRowBytes));
         };
-        // K step ks: its matrix instructions, with the LDS reads of step ks+1's fragments placed one
-        // behind each of the first TN + TM of them. Issued as a block in front of the matrix
-        // instructions, the reads of the two wavefronts of a SIMD and their matrix instructions took
-        // turns instead of overlapping (8 experts x 2560 rows, hidden size 4096: 3.80 against 3.49 ms
-        // for the two projections with the reads interleaved; operands resident in L2: 3.49 against 2.96).
-        auto step = [&](const char* st, int ks) {
-            __builtin_amdgcn_sched_barrier(0);
-            if (ks + 1 < kSteps) read_fragments(st, ks + 1);
+        // Where one load of slice kn comes from and goes to (load li < LA: activation rows, else weight rows).
+        struct SliceLoads { char* sa; char* sb; uint32_t k0; };
+        auto loads_of = [&](uint32_t kn) {
+            SliceLoads l;
+            l.sa = smem + stage_of(t, kn) * kStage;
+            l.sb = l.sa + kABytes;
+            uint32_t slice = kn + t.k_first;
+            slice = slice >= t.k_tiles ? slice - t.k_tiles : slice;
+            l.k0 = slice * BK;
+            return l;
+        };
+        // K step ks in a pinned order: one matrix instruction, behind it one LDS read of step ks+1's
+        // fragments (the first TN + TM instructions) and, with LOADS, one global load of a later slice
+        // (loads load_base, load_base + 1, ... of it), and again. Issued as blocks - all reads, then all
+        // matrix instructions - the two wavefronts of a SIMD took turns instead of overlapping, and a
+        // slice's loads in a block in front of a K step held the matrix cores up (8 experts x 2560
+        // rows, hidden size 4096, both projections: 3.80 ms in blocks, 3.49 with the reads interleaved,
+        // 3.47 with the loads interleaved too; with operands resident in L2 3.49, 2.96 and 2.72).
+        // LOADS is a compile-time switch: a branch around matrix instructions makes the compiler keep
+        // two copies of the accumulators.
+        auto kstep = [&](const char* st, int ks, auto loads_tag, const SliceLoads& l, int load_base) {
+            constexpr bool LOADS = decltype(loads_tag)::value;
 #pragma unroll
-            for (int ni = 0; ni < TN; ++ni)
-#pragma unroll
-                for (int mi = 0; mi < TM; ++mi)
-                    acc[ni][mi] = Elem16<E>::mfma32(fw[ks & 1][ni], fx[ks & 1][mi], acc[ni][mi]);
-            if (ks + 1 < kSteps) {
-#pragma unroll
-                for (int i = 0; i < TN + TM; ++i) {
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // one matrix instruction
-                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // one LDS read
+            for (int i = 0; i < TN * TM; ++i) {
+                __builtin_amdgcn_sched_barrier(0);
+                const int ni = i / TM, mi = i % TM;
+                acc[ni][mi] = Elem16<E>::mfma32(fw[ks & 1][ni], fx[ks & 1][mi], acc[ni][mi]);
+                if (ks + 1 < kSteps) {
+                    const int nb = (ks + 1) & 1;
+                    if (i < TN) fw[nb][i] = __builtin_bit_cast(vec8, load16(st + (base_w ^ ((ks + 1) << 5)) + i * 32 * kRowBytes));
+                    else if (i < TN + TM) fx[nb][i - TN] = __builtin_bit_cast(vec8, load16(st + (base_x ^ ((ks + 1) << 5)) + (i - TN) * 32 * kRowBytes));
+                }
+                if constexpr (LOADS) {
+                    const int li = load_base + i;
+                    if (li < LA)
+                        __builtin_amdgcn_global_load_lds((global_cptr)(t.pa[li] + l.k0), (lds_ptr)(l.sa + 1024 * (wave + kWaves * li)), 16, 0, 0);
+                    else if (li < LA + LB)
+                        __builtin_amdgcn_global_load_lds((global_cptr)(t.pb[li - LA] + l.k0), (lds_ptr)(l.sb + 1024 * (wave + kWaves * (li - LA))), 16,
+                                                         0, STREAM_B ? kNonTemporal : 0);
                 }
             }
-            __builtin_amdgcn_sched_group_barrier(0x008, TN * TM, 0);     // the remaining matrix instructions
             __builtin_amdgcn_sched_barrier(0);
         };
+        constexpr std::true_type with_loads{};
+        constexpr std::false_type without_loads{};
+        static_assert(TN + TM <= TN * TM, "a K step has a matrix instruction for every fragment read");
         if constexpr (AHEAD2) {
+            static_assert(LA + LB <= TN * TM, "the loads of a slice fit behind the matrix instructions of one K step");
             // Slice 0 was requested by begin(). Every wavefront has left the previous tile's epilogue,
             // which staged its output in the stage slice 1 goes to.
             asm volatile("s_barrier" ::: "memory");
             if (t.k_tiles > 1) issue_slice(t, smem, 1);
-            for (uint32_t kt = 0; kt < t.k_tiles; ++kt) {
+            auto top = [&](uint32_t kt) {
                 // this wavefront's loads of slice kt are complete once only those of slice kt+1 are
                 // outstanding (the stores of the previous tile's epilogue are older than both)
                 if (kt + 1 < t.k_tiles) wait_vmcnt<kLoadsPerSlice>();
                 else wait_vmcnt<0>();
                 asm volatile("s_barrier" ::: "memory");   // every wavefront's share of slice kt is in LDS
                 if (kt == 0) after_first_barrier();
+            };
+            const uint32_t ahead = t.k_tiles >= 2 ? t.k_tiles - 2 : 0u;   // slices that request slice kt+2
+            for (uint32_t kt = 0; kt < ahead; ++kt) {
+                top(kt);
                 const char* st = smem + stage_of(t, kt) * kStage;
                 read_fragments(st, 0);
+                const SliceLoads l = loads_of(kt + 2);
 #pragma unroll
-                for (int ks = 0; ks < kSteps; ++ks) {
-                    if (ks == kSteps - 1 && kt + 2 < t.k_tiles) {
-                        // this wavefront's last reads of the stage have returned; once that holds for
-                        // every wavefront the stage takes slice kt+2
-                        __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0)
-                        asm volatile("s_barrier" ::: "memory");
-                        issue_slice(t, smem, kt + 2);
-                    }
-                    step(st, ks);
-                }
+                for (int ks = 0; ks + 1 < kSteps; ++ks) kstep(st, ks, without_loads, l, 0);
+                // this wavefront's last reads of the stage have returned; once that holds for every
+                // wavefront the stage takes slice kt+2
+                __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0)
+                asm volatile("s_barrier" ::: "memory");
+                kstep(st, kSteps - 1, with_loads, l, 0);
+            }
+            for (uint32_t kt = ahead; kt < t.k_tiles; ++kt) {
+                top(kt);
+                const char* st = smem + stage_of(t, kt) * kStage;
+                read_fragments(st, 0);
+                const SliceLoads l{};
+#pragma unroll
+                for (int ks = 0; ks < kSteps; ++ks) kstep(st, ks, without_loads, l, 0);
             }
         } else {
-            for (uint32_t kt = 0; kt < t.k_tiles; ++kt) {
+            static_assert(LA + LB <= kSteps * TN * TM, "the loads of a slice fit behind the matrix instructions of a slice");
+            auto top = [&](uint32_t kt) {
                 // This wavefront's loads of slice kt are complete once only those of the later slices
                 // already issued (STAGES-2 of them, fewer at the end of the tile) are outstanding.
                 const uint32_t later = t.k_tiles - 1 - kt;
@@ -373,13 +408,23 @@ struct Gemm16 {
                 // the next loads overwrite (slice kt-1, or the previous tile's epilogue staging)
                 asm volatile("s_barrier" ::: "memory");
                 if (kt == 0) after_first_barrier();
+            };
+            const uint32_t ahead = t.k_tiles >= uint32_t(STAGES - 1) ? t.k_tiles - (STAGES - 1) : 0u;   // slices that request a later one
+            for (uint32_t kt = 0; kt < ahead; ++kt) {
+                top(kt);
                 const char* st = smem + stage_of(t, kt) * kStage;
                 read_fragments(st, 0);
+                const SliceLoads l = loads_of(kt + STAGES - 1);
 #pragma unroll
-                for (int ks = 0; ks < kSteps; ++ks) {
-                    if (ks == 0 && kt + STAGES - 1 < t.k_tiles) issue_slice(t, smem, kt + STAGES - 1);
-                    step(st, ks);
-                }
+                for (int ks = 0; ks < kSteps; ++ks) kstep(st, ks, with_loads, l, ks * TN * TM);
+            }
+            for (uint32_t kt = ahead; kt < t.k_tiles; ++kt) {
+                top(kt);
+                const char* st = smem + stage_of(t, kt) * kStage;
+                read_fragments(st, 0);
+                const SliceLoads l{};
+#pragma unroll
+                for (int ks = 0; ks < kSteps; ++ks) kstep(st, ks, without_loads, l, 0);
             }
         }
     }
