@@ -19,12 +19,13 @@ namespace kleos_amd {
 // global->LDS loads (global_load_lds_dwordx4: each lane names a 16-byte global source, the 64 lanes
 // of the instruction land in 1 KB of consecutive LDS). They never occupy a vector register. Rows of
 // A are gathered through the slot->token table by giving each lane its token's row address.
-// Slice kt+STAGES-1 is requested at the start of slice kt, into the stage slice kt-1 was read from.
+// Slice kt+STAGES-1 is requested during slice kt, into the stage slice kt-1 was read from, its loads
+// placed one by one behind the matrix instructions of the slice's first K steps.
 // With two stages the loads can instead run two slices ahead (AHEAD2): slice kt+2 is requested
 // into the stage of slice kt as soon as every wavefront has read its last fragments of slice kt (a
-// second workgroup barrier per slice, placed before the last group of matrix instructions), so the
-// memory pipeline holds requests across the wait for slice kt+1 instead of running empty at
-// every slice boundary.
+// second workgroup barrier per slice, placed before the last K step, whose matrix instructions
+// the loads then follow one by one), so the memory pipeline holds requests across the wait for
+// slice kt+1 instead of running empty at every slice boundary.
 //
 // LDS layout of a stage: rows of BK*2 bytes, 16-byte chunk c of row r stored at chunk position
 // c ^ swizzle(r). The LDS of gfx950 has 64 banks of 4 bytes and serves a 16-byte access of 16 lanes

@@ -42,7 +42,7 @@ constexpr int kXcds = 8;
 // leave room for a third one (measured on the 256-expert top-8 shape: 3.7 ms against 4.6 ms).
 // Variant 2, for layers whose experts hold at least four row blocks (few large experts: every
 // weight tile is shared by several workgroups through L2, loads return quickly and the matrix work
-// dominates): the tile of variant 0 with the loads one slice ahead, issued at the first K step.
+// dominates): the tile of variant 0 with the loads one slice ahead, issued during the first K step.
 // Variants 0 and 1 load their weight rows non-temporally (headline 378 against 390 us per forward,
 // the 16-expert shape 192 against 196, the 256-expert shape 3.43 against 3.48 ms); variant 2, whose
 // weight tiles are shared by eight workgroups and more, does not (4.06 against 4.01 ms with it).
