@@ -108,11 +108,26 @@ __device__ __forceinline__ void atomic_store_relaxed(uint32_t* p, uint32_t v) {
     __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// Device-coherent reads of data another workgroup of the same launch wrote (and made visible with
-// a device-scope release). The eight L2 caches of the device are not coherent with each other, and
-// a line read in an earlier phase or launch may still sit in this XCD's L2: these loads carry the
-// agent scope (sc1), which the caches do not serve from such a line. Reading the few tables that
-// cross workgroups this way replaces invalidating the whole L2 after every grid-wide barrier.
+// Data that crosses workgroups inside one launch. The eight L2 caches of the device are not
+// coherent with each other: a plain store may stay in the writer's L2, and a line read in an
+// earlier phase or launch may still sit in the reader's. Writing such data back with a
+// device-scope release and dropping stale lines with a device-scope acquire walks a whole L2 each
+// time (about 2 us per release at a grid-wide barrier, tens of microseconds of refetching per
+// acquire), so the tables and rows that cross workgroups are instead written and read with the
+// agent scope (sc1) on the instructions themselves:
+//   * store_through / store16_through / the sc1 buffer stores of the GEMM epilogue write through
+//     the L2 to memory; once the wavefront's vmcnt has drained they are visible device-wide, which
+//     is all a grid-wide barrier or a readiness counter has to wait for;
+//   * load_coherent / load16_coherent are not served from a stale line.
+template <typename V, typename U>
+__device__ __forceinline__ void store_through(V* p, U v) {
+    static_assert(sizeof(V) == 4 || sizeof(V) == 8);
+    __hip_atomic_store(p, static_cast<V>(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// 16 bytes at a per-lane address (16-byte aligned).
+__device__ __forceinline__ void store16_through(void* p, u32x4 v) {
+    asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(p), "v"(v) : "memory");
+}
 template <typename V>
 __device__ __forceinline__ V load_coherent(const V* p) {
     static_assert(sizeof(V) == 4 || sizeof(V) == 8);

@@ -93,11 +93,12 @@ __device__ __forceinline__ uint32_t local_tid() {
 // lines of the output rows. The bias comes from LDS (bias_mem: the tile's BN entries): the epilogue
 // issues no global load, so nothing in it ever waits for the stores it has in flight.
 constexpr int kEpiloguePanelRows = 32;
-// THROUGH: the output rows are stored with the agent-scope (sc1) policy, which writes them through
-// the L2 instead of leaving dirty lines there. It pays where a launch writes far more output than
-// the L2 holds and nothing on the same XCD reads it back soon (256-expert top-8 shape: 3.03
+// The output rows are stored with the agent-scope (sc1) policy, which writes them through the L2
+// instead of leaving dirty lines there: other workgroups read them later in the same launch, on
+// any XCD, and nothing then has to write a whole L2 back before it may tell them so. It also pays
+// by itself where a launch writes far more output than the L2 holds (256-expert top-8 shape: 3.03
 // against 3.11 ms per forward); neutral on the other shapes measured.
-template <typename E, int WM, int WN, int WAVES_N, int ACT, bool THROUGH>
+template <typename E, int WM, int WN, int WAVES_N, int ACT>
 __device__ __forceinline__ void epilogue16_act(const TileOut& t, f32x16 (&acc)[WN / 32][WM / 32], char* stage_mem,
                                                const char* bias_mem) {
     typedef typename Elem16<E>::vec4 vec4;
@@ -134,25 +135,21 @@ __device__ __forceinline__ void epilogue16_act(const TileOut& t, f32x16 (&acc)[W
                 const u32x4 v = load16(stg + r * 128 + ((c ^ ((r >> 1) & 7)) << 4));
                 const uint32_t m = wm * WM + mi * 32 + r, n = wn * WN + pn * 64 + c * 8;
                 if (m < t.m_valid && n < t.n_valid) {
-                    if constexpr (THROUGH) {
-                        constexpr int kAgentScope = 16;   // sc1
-                        // (a tile's rows lie within 2 GiB of its first element: 256 rows of at most 2^22 bytes)
-                        __builtin_amdgcn_raw_buffer_store_b128(v, coherent_rows(t.c_base), int((size_t(m) * t.ldc + n) * sizeof(E)), 0,
-                                                               kAgentScope);
-                    } else {
-                        store16(t.c_base + size_t(m) * t.ldc + n, v);
-                    }
+                    constexpr int kAgentScope = 16;   // sc1
+                    // (a tile's rows lie within 2 GiB of its first element: 256 rows of at most 2^22 bytes)
+                    __builtin_amdgcn_raw_buffer_store_b128(v, coherent_rows(t.c_base), int((size_t(m) * t.ldc + n) * sizeof(E)), 0,
+                                                           kAgentScope);
                 }
             }
         }
     }
 }
-template <typename E, int WM, int WN, int WAVES_N, bool THROUGH>
+template <typename E, int WM, int WN, int WAVES_N>
 __device__ __forceinline__ void epilogue16(const TileOut& t, f32x16 (&acc)[WN / 32][WM / 32], char* stage_mem,
                                            const char* bias_mem) {
-    if (t.act == 0) epilogue16_act<E, WM, WN, WAVES_N, 0, THROUGH>(t, acc, stage_mem, bias_mem);
-    else if (t.act == 1) epilogue16_act<E, WM, WN, WAVES_N, 1, THROUGH>(t, acc, stage_mem, bias_mem);
-    else epilogue16_act<E, WM, WN, WAVES_N, 2, THROUGH>(t, acc, stage_mem, bias_mem);
+    if (t.act == 0) epilogue16_act<E, WM, WN, WAVES_N, 0>(t, acc, stage_mem, bias_mem);
+    else if (t.act == 1) epilogue16_act<E, WM, WN, WAVES_N, 1>(t, acc, stage_mem, bias_mem);
+    else epilogue16_act<E, WM, WN, WAVES_N, 2>(t, acc, stage_mem, bias_mem);
 }
 
 // STREAM_B: the weight rows are loaded with the non-temporal cache policy: read once (or by a
@@ -163,8 +160,7 @@ __device__ __forceinline__ void epilogue16(const TileOut& t, f32x16 (&acc)[WN / 
 // its matrix work (headline shape: 301 against 315 us for the expert phase); where the matrix work
 // dominates the extra barrier costs more than the earlier loads bring (8-expert shape with hidden
 // size 4096: 4.22 against 4.03 ms).
-// THROUGH_C: the epilogue writes the output rows through the L2 (see epilogue16_act).
-template <typename E, int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES, bool STREAM_B, bool AHEAD2, bool THROUGH_C = false>
+template <typename E, int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES, bool STREAM_B, bool AHEAD2>
 struct Gemm16 {
     typedef typename Elem16<E>::vec8 vec8;
     typedef typename Elem16<E>::vec4 vec4;
@@ -461,7 +457,8 @@ struct Gemm16 {
                     const int r = id >> 3, c = id & 7;
                     const u32x4 v = load16(stg + r * 128 + ((c ^ ((r >> 1) & 7)) << 4));
                     const uint32_t m = wm * WM + mi * 32 + r, n = wn * WN + ni * 32 + c * 4;
-                    if (m < t.m_valid && n < t.n_valid) store16(out + size_t(m) * ldo + n, v);
+                    // the sums are read by other workgroups after a grid-wide barrier
+                    if (m < t.m_valid && n < t.n_valid) store16_through(out + size_t(m) * ldo + n, v);
                 }
             }
     }
@@ -469,7 +466,7 @@ struct Gemm16 {
     // Epilogue. Every wavefront must have left mainloop().
     static __device__ __forceinline__ void finish(const Tile& t, Acc& acc, char* smem) {
         const TileOut out{t.c_base, t.ldc, t.m_valid, t.n_valid, t.act};
-        epilogue16<E, WM, WN, WAVES_N, THROUGH_C>(out, acc, smem + last_stage(t) * kStage, smem + kBiasOffset + t.bias_slot * kBiasBytes);
+        epilogue16<E, WM, WN, WAVES_N>(out, acc, smem + last_stage(t) * kStage, smem + kBiasOffset + t.bias_slot * kBiasBytes);
     }
 };
 
@@ -535,7 +532,8 @@ __device__ __forceinline__ void gemm_tile_f32(
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const uint32_t n = tx * 4 + j;
-            if (n < n_valid) c_base[size_t(m) * ldc + n] = activate<ACT>(acc[i][j] + bias[n]);
+            // read by other workgroups later in the same launch: written through the L2
+            if (n < n_valid) store_through(c_base + size_t(m) * ldc + n, activate<ACT>(acc[i][j] + bias[n]));
         }
     }
 }

@@ -13,6 +13,8 @@
 //     makes dropping deterministic; the reference takes a tile's base slot from atomicAdd arrival
 //     order (gate.cuh:699).
 #pragma once
+#include <type_traits>
+
 #include "device_common.hpp"
 
 namespace kleos_amd {
@@ -31,10 +33,25 @@ struct GateK {
 template <int NG>
 constexpr int gate_unit_blocks() { return NG == 0 || NG >= 16 ? 1 : 2; }
 
-// LDS floats needed by gate_unit with KW wavefronts: the partial accumulators (4*NG registers of
-// 64 lanes) of the KW shares of the hidden dimension of the block being reduced.
+__host__ __device__ inline uint32_t gate_group_words(uint32_t E, uint32_t k, bool training);
+// Softmax, top-k, outputs and histogram of a 16-token tile by a group of four wavefronts (below).
+template <typename T, int NL>
+__device__ __forceinline__ void gate_group_finish(const LayerParams& p, uint32_t tile, bool valid, f32x4 (&acc)[NL], uint32_t* gsm, uint32_t gtid);
+// Up to 64 experts (four groups) and a multiple of four wavefronts: the epilogue of a block is
+// shared out over a group of four wavefronts instead of run by one.
 template <int NG>
-constexpr int gate_smem_floats(int kw) { return kw * (NG == 0 ? 16 : NG) * 4 * kWave; }
+constexpr bool gate_unit_grouped(int kw) { return NG >= 1 && NG <= 4 && kw % 4 == 0; }
+// Row stride of the parked partial sums in the grouped epilogue: one word more than a wavefront
+// writes, so that the reads, which walk the rows four at a time, spread over all banks.
+constexpr int kGateParkStride = kWave + 1;
+// LDS floats needed by gate_unit with KW wavefronts: the partial accumulators (4*NG registers of
+// 64 lanes) of the KW shares of the hidden dimension of the block being reduced; in the grouped
+// epilogue those of both blocks, in padded rows, and the scratch of the groups.
+template <int NG>
+constexpr int gate_smem_floats(int kw) {
+    if (gate_unit_grouped<NG>(kw)) return 2 * kw * NG * 4 * kGateParkStride + (kw / 4) * int(kGateTileTokens * 64 + 64 + kGateTileTokens * 64);
+    return kw * (NG == 0 ? 16 : NG) * 4 * kWave;
+}
 constexpr uint32_t kWideGateMaxK = 32;   // the wide gate keeps a tile's 16 * k picks in LDS
 
 // Softmax, top-k, outputs and the tile histogram of one 16-token tile, run by one wavefront that
@@ -100,7 +117,7 @@ __device__ __forceinline__ void gate_epilogue(const LayerParams& p, uint32_t til
                 col_sum += __shfl_xor(col_sum, 2);
                 col_sum += __shfl_xor(col_sum, 4);
                 col_sum += __shfl_xor(col_sum, 8);
-                if (col == 0 && e < E) p.tile_prob[size_t(tile) * E + e] = col_sum;
+                if (col == 0 && e < E) store_through(p.tile_prob + size_t(tile) * E + e, col_sum);
             }
     }
 
@@ -151,11 +168,11 @@ __device__ __forceinline__ void gate_epilogue(const LayerParams& p, uint32_t til
         pv += __shfl_xor(pv, 32);
         den += pv;   // mCw, accumulated in selection order (gate.cuh:669)
         if (chunk == 0) {
-            p.topk_expert[size_t(token) * p.k + r] = int32_t(bi);
-            p.topk_prob[size_t(token) * p.k + r] = pv;
+            store_through(p.topk_expert + size_t(token) * p.k + r, int32_t(bi));
+            store_through(p.topk_prob + size_t(token) * p.k + r, pv);
         }
     }
-    if (chunk == 0) p.combine_den[token] = den;
+    if (chunk == 0) store_through(p.combine_den + token, den);
 
     // Histogram of the tile and each token's rank inside it (gate.cuh:678-696).
     uint32_t* super = p.super_count + size_t(p.epoch & 1u) * p.n_super * E +
@@ -170,10 +187,10 @@ __device__ __forceinline__ void gate_epilogue(const LayerParams& p, uint32_t til
             const unsigned long long mask = __ballot(sel);
             const uint32_t sub = uint32_t(mask >> (16 * chunk)) & 0xffffu;
             if (sel)
-                p.topk_slot[size_t(token) * p.k + (rnd - 1)] = int32_t(__popc(sub & ((1u << col) - 1u)));
+                store_through(p.topk_slot + size_t(token) * p.k + (rnd - 1), int32_t(__popc(sub & ((1u << col) - 1u))));
             if (col == 0 && e < E) {
                 const uint32_t cnt = __popc(sub);
-                p.tile_count[size_t(tile) * E + e] = cnt;
+                store_through(p.tile_count + size_t(tile) * E + e, cnt);
                 if (cnt) atomic_add_agent(super + e, cnt);
             }
         }
@@ -256,6 +273,47 @@ __device__ __forceinline__ void gate_unit(const LayerParams& p, uint32_t unit, f
         }
     }
 
+    if constexpr (gate_unit_grouped<NG>(KW)) {
+        // Every wavefront parks the partial sums of its share of both blocks in LDS; block b then
+        // belongs to group b of four wavefronts (one group: block after block), 16 lanes per token
+        // and four experts per lane, which add the shares in ascending order (a fixed order: the
+        // logits depend neither on timing nor on which wavefront worked on which share).
+        static_assert(TB == 2);
+        constexpr int kShare = NG * 4 * kGateParkStride;
+#pragma unroll
+        for (int b = 0; b < TB; ++b) {
+            float* dst = smem + (b * KW + part) * kShare;
+#pragma unroll
+            for (int g = 0; g < NG; ++g)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) dst[(g * 4 + v) * kGateParkStride + lane] = acc[b][g][v];
+        }
+        __syncthreads();
+        constexpr int kGroups = KW / 4;
+        const uint32_t group = uint32_t(wave) >> 2, gtid = threadIdx.x & 255u;
+        uint32_t* gsm = reinterpret_cast<uint32_t*>(smem + TB * KW * kShare) + group * gate_group_words(p.E, p.k, p.is_training != 0);
+        const int sub = lane & 15;                              // experts 4 sub .. 4 sub + 3
+        const int tl = 4 * (wave & 3) + (lane >> 4);            // token inside the block
+#pragma unroll
+        for (int b0 = 0; b0 < TB; b0 += kGroups) {
+            const uint32_t b = b0 + group;
+            const uint32_t tile = unit * TB + b;
+            const bool valid = b < uint32_t(TB) && tile < p.n_gate_tiles;
+            f32x4 sum[1] = {f32x4{0.f, 0.f, 0.f, 0.f}};
+            if (valid && sub < 4 * NG) {
+                // expert 4 sub + v sits in row 4 (sub / 4) + v of a share, at lane 16 (sub % 4) + token
+                const float* src = smem + (b * KW) * kShare + ((sub >> 2) * 4) * kGateParkStride + 16 * (sub & 3) + tl;
+#pragma unroll
+                for (int v = 0; v < 4; ++v) sum[0][v] = src[v * kGateParkStride];
+#pragma unroll
+                for (int w = 1; w < KW; ++w)
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) sum[0][v] += src[w * kShare + v * kGateParkStride];
+            }
+            gate_group_finish<T, 1>(p, tile, valid, sum, gsm, gtid);
+        }
+        return;
+    }
     // Block b: every wavefront parks the partial sums of its share in LDS, wavefront b adds them
     // in ascending order of the shares (a fixed order: the logits depend neither on timing nor on
     // which wavefront worked on which share).
@@ -424,7 +482,7 @@ __device__ __forceinline__ void gate_wide_epilogue(const LayerParams& p, uint32_
                     col_sum += __shfl_xor(col_sum, 2);
                     col_sum += __shfl_xor(col_sum, 4);
                     col_sum += __shfl_xor(col_sum, 8);
-                    if (col == 0 && e < E) p.tile_prob[size_t(tile) * E + e] = col_sum;
+                    if (col == 0 && e < E) store_through(p.tile_prob + size_t(tile) * E + e, col_sum);
                 }
             }
 
@@ -464,12 +522,12 @@ __device__ __forceinline__ void gate_wide_epilogue(const LayerParams& p, uint32_
             prev_l = best;
             prev_e = bi;
             if (chunk == 0) {
-                p.topk_expert[size_t(token) * k + r] = int32_t(bi);
-                p.topk_prob[size_t(token) * k + r] = pv;
+                store_through(p.topk_expert + size_t(token) * k + r, int32_t(bi));
+                store_through(p.topk_prob + size_t(token) * k + r, pv);
                 s_sel[uint32_t(col) * k + r] = bi;
             }
         }
-        if (chunk == 0) p.combine_den[token] = den;
+        if (chunk == 0) store_through(p.combine_den + token, den);
         // in-tile rank of every pick and the tile histogram (gate.cuh:678-696); the LDS operations of
         // one wavefront complete in order, so the picks written above are visible here
         uint32_t* super = p.super_count + size_t(p.epoch & 1u) * p.n_super * E + size_t(tile / kSuperTiles) * E;
@@ -482,12 +540,12 @@ __device__ __forceinline__ void gate_wide_epilogue(const LayerParams& p, uint32_
                 total += same;
                 before += same && o / k < t;
             }
-            p.topk_slot[(size_t(tile) * kGateTileTokens + t) * k + (i % k)] = int32_t(before);
+            store_through(p.topk_slot + ((size_t(tile) * kGateTileTokens + t) * k + (i % k)), int32_t(before));
             if (before == 0 && e < E) s_hist[e] = total;   // one writer: the first token that picked e
         }
         for (uint32_t e = lane; e < E; e += kWave) {
             const uint32_t cnt = s_hist[e];
-            p.tile_count[size_t(tile) * E + e] = cnt;
+            store_through(p.tile_count + size_t(tile) * E + e, cnt);
             if (cnt) atomic_add_agent(super + e, cnt);
         }
     }
@@ -519,9 +577,9 @@ __device__ __forceinline__ f32x4 gate_partial_sum(const LayerParams& p, coherent
 // the group takes tokens 4 w .. 4 w + 3 of the tile, 16 lanes per token, each lane the experts
 // 64 j + 4 (lane % 16) + v (j < NL, NL * 64 >= PX, v < 4). Against one wavefront per tile every per-lane
 // loop over the experts is four times shorter, and the partial sums, logits and gate outputs move
-// in runs of 256 and 128 bytes per token. The tile's picks meet in LDS: one wavefront assigns the
-// in-tile ranks token by token (a token's k experts are distinct, so the lanes of a step never
-// touch the same histogram word), then the group writes the histogram out. Same sums over the
+// in runs of 256 and 128 bytes per token. The tile's picks meet in LDS: every pick counts the picks
+// of its expert by earlier tokens for its in-tile rank and adds itself to the tile's histogram,
+// which the group then writes out. Same sums over the
 // ranges, same selection rule and same order of the denominator as gate_epilogue; the softmax
 // denominator is summed in a different (fixed) order.
 // `gsm`: gate_group_words(p) words of LDS private to the group. Every thread of the workgroup must
@@ -532,20 +590,14 @@ __host__ __device__ inline uint32_t gate_group_words(uint32_t E, uint32_t k, boo
 }
 template <typename T, int NL>
 __device__ __forceinline__ void gate_reduce_group(const LayerParams& p, uint32_t tile, bool valid, uint32_t* gsm, uint32_t gtid) {
-    constexpr uint32_t kGroupThreads = 4 * kWave;
     const int lane = gtid & 63, sub = lane & 15;
-    const uint32_t gw = gtid >> 6, tl = 4 * gw + (lane >> 4);
-    const uint32_t E = p.E, k = p.k;
-    uint32_t* s_sel = gsm;                                   // [16][k] expert picked by token t in round r
-    uint32_t* s_hist = gsm + kGateTileTokens * k;            // [E]
-    float* s_prob = reinterpret_cast<float*>(s_hist + E);    // [16][E], training only
-    for (uint32_t e = gtid; e < E; e += kGroupThreads) s_hist[e] = 0u;
+    const uint32_t tl = 4 * (gtid >> 6) + (lane >> 4);
+    f32x4 acc[NL];
+#pragma unroll
+    for (int j = 0; j < NL; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
     if (valid) {
         const uint32_t token = tile * kGateTileTokens + tl;
         const coherent_rows_t partial = coherent_rows(p.gate_partial);
-        f32x4 acc[NL];
-#pragma unroll
-        for (int j = 0; j < NL; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
         // range by range, in ascending order; the loads of two ranges in flight together
         for (uint32_t s0 = 0; s0 < p.gate_splits; s0 += 2) {
             u32x4 v[2][NL];
@@ -563,17 +615,39 @@ __device__ __forceinline__ void gate_reduce_group(const LayerParams& p, uint32_t
                 for (int j = 0; j < NL; ++j) acc[j] += __builtin_bit_cast(f32x4, v[1][j]);
             }
         }
+    }
+    gate_group_finish<T, NL>(p, tile, valid, acc, gsm, gtid);
+}
+
+// The part of the group's work that follows the logits: `acc[j][v]` of a lane is the logit of expert
+// 64 j + 4 (lane % 16) + v of its token (anything for experts past the padded count).
+template <typename T, int NL>
+__device__ __forceinline__ void gate_group_finish(const LayerParams& p, uint32_t tile, bool valid, f32x4 (&acc)[NL], uint32_t* gsm, uint32_t gtid) {
+    constexpr uint32_t kGroupThreads = 4 * kWave;
+    const int lane = gtid & 63, sub = lane & 15;
+    const uint32_t gw = gtid >> 6, tl = 4 * gw + (lane >> 4);
+    const uint32_t E = p.E, k = p.k;
+    uint32_t* s_sel = gsm;                                   // [16][k] expert picked by token t in round r
+    uint32_t* s_hist = gsm + kGateTileTokens * k;            // [E]
+    float* s_prob = reinterpret_cast<float*>(s_hist + E);    // [16][E], training only
+    for (uint32_t e = gtid; e < E; e += kGroupThreads) s_hist[e] = 0u;
+    if (valid) {
+        const uint32_t token = tile * kGateTileTokens + tl;
         const float kNegInf = -__builtin_inff();
         float m = kNegInf;
+        const bool whole_quads = (E & 3u) == 0u;   // a lane's four experts are all real or all padding
 #pragma unroll
-        for (int j = 0; j < NL; ++j)
+        for (int j = 0; j < NL; ++j) {
+            const uint32_t e0 = 64 * j + 4 * sub;
+            if (whole_quads && e0 < E) *reinterpret_cast<f32x4*>(p.logits + size_t(token) * E + e0) = acc[j];
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
-                const uint32_t e = 64 * j + 4 * sub + v;
-                if (e < E) p.logits[size_t(token) * E + e] = acc[j][v];
-                else acc[j][v] = kNegInf;   // softmax domain = the E real experts only (gate.cuh:550)
+                const uint32_t e = e0 + v;
+                if (e >= E) acc[j][v] = kNegInf;   // softmax domain = the E real experts only (gate.cuh:550)
+                else if (!whole_quads) p.logits[size_t(token) * E + e] = acc[j][v];
                 m = fmaxf(m, acc[j][v]);
             }
+        }
 #pragma unroll
         for (int off = 1; off <= 8; off <<= 1) m = fmaxf(m, __shfl_xor(m, off));
         float d = 0.f;
@@ -596,10 +670,12 @@ __device__ __forceinline__ void gate_reduce_group(const LayerParams& p, uint32_t
                 o[v] = float_to_elem<T>(e < E ? prob(acc[j][v]) : 0.f);
                 if (p.is_training && e < E) s_prob[tl * E + e] = prob(acc[j][v]);
             }
-            static_assert(sizeof(T) == 2);
-            uint2 raw;
-            __builtin_memcpy(&raw, o, 8);
-            if (uint32_t(64 * j) < p.PX) *reinterpret_cast<uint2*>(grow + 64 * j + 4 * sub) = raw;
+            // the padded row length is a multiple of 64: the four columns are inside the row together
+            using Quad = std::conditional_t<sizeof(T) == 2, uint2, f32x4>;
+            static_assert(sizeof(Quad) == 4 * sizeof(T));
+            Quad raw;
+            __builtin_memcpy(&raw, o, sizeof(Quad));
+            if (uint32_t(64 * j) < p.PX) *reinterpret_cast<Quad*>(grow + 64 * j + 4 * sub) = raw;
         }
         // top-k: k rounds of arg-max, equal values go to the lower expert index (gate.cuh:654-670);
         // a picked expert leaves the working copy
@@ -637,39 +713,47 @@ __device__ __forceinline__ void gate_reduce_group(const LayerParams& p, uint32_t
                 for (int v = 0; v < 4; ++v)
                     if (uint32_t(64 * j + 4 * sub + v) == bi) w[j][v] = kNegInf;
             if (sub == 0) {
-                p.topk_expert[size_t(token) * k + r] = int32_t(bi);
-                p.topk_prob[size_t(token) * k + r] = pv;
+                store_through(p.topk_expert + size_t(token) * k + r, int32_t(bi));
+                store_through(p.topk_prob + size_t(token) * k + r, pv);
                 s_sel[tl * k + r] = bi;
             }
         }
-        if (sub == 0) p.combine_den[token] = den;
+        if (sub == 0) store_through(p.combine_den + token, den);
     }
     __syncthreads();
-    // in-tile ranks (gate.cuh:678-696): token by token; LDS operations of one wavefront complete in order
-    if (valid && gw == 0) {
-        for (uint32_t t = 0; t < kGateTileTokens; ++t)
-            for (uint32_t r = lane; r < k; r += kWave) {
-                const uint32_t e = s_sel[t * k + r];
-                uint32_t rank = 0;
-                if (e < E) {
-                    rank = s_hist[e];
-                    s_hist[e] = rank + 1u;
+    // in-tile ranks (gate.cuh:678-696): pick r of token t ranks behind the picks of the same expert
+    // by the tokens before t (a token's own picks are distinct experts). One pick per thread, the
+    // earlier picks read four at a time (every lane reads the same words: broadcasts); the reads
+    // may run up to three words past the picks of the earlier tokens, which stays inside the
+    // group's LDS and is masked out.
+    if (valid) {
+        for (uint32_t i = gtid; i < kGateTileTokens * k; i += kGroupThreads) {
+            const uint32_t e = s_sel[i];
+            const uint32_t before = (i / k) * k;
+            uint32_t rank = 0;
+            if (e < E) {
+                for (uint32_t j = 0; j < before; j += 4) {
+                    const uint32_t a = s_sel[j], b = s_sel[j + 1], c = s_sel[j + 2], d = s_sel[j + 3];
+                    rank += uint32_t(a == e) + uint32_t(b == e && j + 1 < before) + uint32_t(c == e && j + 2 < before) +
+                            uint32_t(d == e && j + 3 < before);
                 }
-                p.topk_slot[(size_t(tile) * kGateTileTokens + t) * k + r] = int32_t(rank);
+                atomicAdd(s_hist + e, 1u);
             }
+            store_through(p.topk_slot + size_t(tile) * kGateTileTokens * k + i, int32_t(rank));
+        }
     }
     __syncthreads();
     if (valid) {
         uint32_t* super = p.super_count + size_t(p.epoch & 1u) * p.n_super * E + size_t(tile / kSuperTiles) * E;
         for (uint32_t e = gtid; e < E; e += kGroupThreads) {
             const uint32_t cnt = s_hist[e];
-            p.tile_count[size_t(tile) * E + e] = cnt;
+            store_through(p.tile_count + size_t(tile) * E + e, cnt);
             if (cnt) atomic_add_agent(super + e, cnt);
             if (p.is_training) {
                 // column sums of the tile's probabilities for the load-balancing loss (gate.cuh:608-635)
                 float col_sum = 0.f;
                 for (uint32_t t = 0; t < kGateTileTokens; ++t) col_sum += s_prob[t * E + e];
-                p.tile_prob[size_t(tile) * E + e] = col_sum;
+                store_through(p.tile_prob + size_t(tile) * E + e, col_sum);
             }
         }
     }
@@ -752,11 +836,11 @@ __device__ __forceinline__ void slot_tile(const LayerParams& p, uint32_t tile, b
 #pragma unroll
                     for (uint32_t u = 0; u < 16; ++u) total += r0 + u < rows ? v[u] : 0.f;
                 }
-                p.super_prob[size_t(sup) * E + e] = total;
+                store_through(p.super_prob + size_t(sup) * E + e, total);
             }
             // total routed per expert, dropped tokens included (the reference's eC, gate.cuh:699)
             if (tile + 1 == p.n_gate_tiles)
-                p.expert_count[e] = acc + load_coherent(p.tile_count + size_t(tile) * E + e);
+                store_through(p.expert_count + e, acc + load_coherent(p.tile_count + size_t(tile) * E + e));
         }
     }
     __syncthreads();
@@ -767,8 +851,8 @@ __device__ __forceinline__ void slot_tile(const LayerParams& p, uint32_t tile, b
             if (e >= E) e = E - 1;   // cannot happen; keeps every address below inside its table
             const uint32_t slot = base[e] + uint32_t(rank);
             const bool keep = slot < p.EC && slot < p.cap_rows;
-            p.topk_slot[idx] = keep ? int32_t(slot) : -1;
-            if (keep) p.slot_token[size_t(e) * p.cap_rows + slot] = int32_t(token);
+            store_through(p.topk_slot + idx, keep ? int32_t(slot) : -1);
+            if (keep) store_through(p.slot_token + size_t(e) * p.cap_rows + slot, int32_t(token));
         };
 #pragma unroll
         for (uint32_t u = 0; u < kInline; ++u)

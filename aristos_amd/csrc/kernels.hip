@@ -46,11 +46,9 @@ constexpr int kXcds = 8;
 // Variants 0 and 1 load their weight rows non-temporally (headline 378 against 390 us per forward,
 // the 16-expert shape 192 against 196, the 256-expert shape 3.43 against 3.48 ms); variant 2, whose
 // weight tiles are shared by eight workgroups and more, does not (4.06 against 4.01 ms with it).
-// Variant 1 also writes its output rows through the L2 (the 256-expert shape stores 0.58 GB per
-// launch: 3.03 against 3.11 ms per forward; no difference on the shapes of variants 0 and 2).
 template <typename E, int V>
 using GemmCfg = std::conditional_t<V == 0, Gemm16<E, 256, 256, 2, 4, 64, 2, true, true>,
-                std::conditional_t<V == 1, Gemm16<E, 128, 256, 2, 4, 64, 3, true, false, true>, Gemm16<E, 256, 256, 2, 4, 64, 2, false, false>>>;
+                std::conditional_t<V == 1, Gemm16<E, 128, 256, 2, 4, 64, 3, true, false>, Gemm16<E, 256, 256, 2, 4, 64, 2, false, false>>>;
 constexpr int kBN = 256;
 constexpr int kGemmThreads = GemmCfg<bf16_t, 0>::kThreads;
 static_assert(GemmCfg<bf16_t, 1>::kThreads == kGemmThreads && GemmCfg<bf16_t, 2>::kThreads == kGemmThreads,
@@ -148,8 +146,11 @@ __device__ __forceinline__ void bounded_wait(uint32_t* sched, unsigned long long
 // wait. The arrival and the wait are the business of the first lane of the last wavefront, so that
 // the wavefronts `between` keeps busy (it may hold workgroup barriers) do not sit behind the
 // arrival's trips to memory longer than they must.
-// Every wavefront first waits for its own outstanding stores: the workgroup barrier does not, and
-// the leader's release covers only what has left the other wavefronts' queues by then.
+// Every wavefront first waits for its own outstanding stores. Whatever another workgroup reads
+// after the barrier was written through the L2 (store_through and the like), so a store that has
+// been acknowledged is visible device-wide and the arrival needs no device-scope release, which
+// would write the whole L2 back (measured: 2 us per barrier and 11-19 us per forward at the
+// 64-expert shape, the other workgroups of the XCD slowed down included).
 template <typename Between>
 __device__ __forceinline__ void grid_barrier(uint32_t* sched, unsigned long long ticks, uint32_t which, uint32_t seq, uint32_t nwg,
                                              Between&& between) {
@@ -161,9 +162,11 @@ __device__ __forceinline__ void grid_barrier(uint32_t* sched, unsigned long long
         const uint32_t members = (nwg - g + kXcds - 1) / kXcds;
         uint32_t* all = sched + kSchedBar + which * kSchedLine;
         uint32_t* mine = sched + kSchedGroup + (which * kXcds + g) * kSchedLine;
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+        // (the workgroup-scope fences keep the compiler from moving memory operations across the
+        // arrivals; the hardware side is the drained vmcnt above)
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         if (atomic_add_agent(mine, 1u) + 1u == (seq + 1u) * members) {
-            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "agent");
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");
             atomic_add_agent(all, 1u);
         }
     }
@@ -175,7 +178,7 @@ __device__ __forceinline__ void grid_barrier(uint32_t* sched, unsigned long long
         bounded_wait(sched, ticks, [&] { return int32_t(atomic_load_relaxed(all) - target) >= 0; });
     }
     __syncthreads();
-    // No device-scope acquire here: it would invalidate the whole L2 of the XCD (tens of
+    // No device-scope acquire here either: it would invalidate the whole L2 of the XCD (tens of
     // microseconds of refetching per launch). What crosses workgroups after a barrier is read
     // with device-coherent loads instead; this only drops the CU's own L1.
     asm volatile("buffer_inv sc0" ::: "memory");
@@ -281,10 +284,6 @@ struct Readiness {
     uint32_t* sched;      // nullptr: no cross-tile dependencies inside this launch (phased mode)
     uint32_t mt_max, tn_up;
     unsigned long long ticks;   // bound of a wait for a row block
-    // Every tile of a queue runs on the queue's own XCD (static schedule): a finished tile is in that
-    // XCD's L2 as soon as its stores are acknowledged, and its readers sit behind the same L2, so
-    // announcing it needs no write-back of the L2. With stealing a reader may sit anywhere.
-    bool local_only;
     __device__ __forceinline__ uint32_t* counter(const Task& t) const { return sched + kSchedReady + t.e * mt_max + t.mtile; }
     // A counter holds the stored tiles of the row block in its low half and, in its high half, how
     // many of them were stored by a workgroup on a foreign XCD (from whose L2 they were written back
@@ -339,11 +338,12 @@ __device__ __forceinline__ void expert_loop(const LayerParams& p, char* smem, ui
         else asm volatile("buffer_inv sc0" ::: "memory");
     };
     auto publish = [&](const Task& t) {
-        // all stores of the tile are complete in every wavefront; make them visible to whoever may
-        // read them, then count the tile (the reference's tQS increment, processor.cuh:719)
+        // all stores of the tile are complete in every wavefront, and they were written through the
+        // L2: the rows are visible to whoever may read them. Count the tile (the reference's tQS
+        // increment, processor.cuh:719)
         if (rd.sched && t.kind == 0 && tid == 0) {
             const unsigned long long t0 = wall_clock64();
-            if (!rd.local_only || t.foreign) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
             atomic_add_agent(rd.counter(t), t.foreign ? 1u + Readiness::kForeignUnit : 1u);
             st_pub += wall_clock64() - t0;
         }
@@ -566,7 +566,7 @@ __global__ __launch_bounds__((TileShape<T, V>::kThreads), (TileShape<T, V>::kPer
         }
         return broadcast_task(s_task, t);
     };
-    expert_loop<T, V>(p, gemm_smem + kPhasedGemmHeader, s_task, Readiness{nullptr, 0, 0, 0, true}, nullptr, next);
+    expert_loop<T, V>(p, gemm_smem + kPhasedGemmHeader, s_task, Readiness{nullptr, 0, 0, 0}, nullptr, next);
 }
 
 template <typename T>
@@ -603,11 +603,13 @@ __global__ __launch_bounds__((TileShape<T, V>::kThreads), (TileShape<T, V>::kPer
     // ---- phase 0: gate. Workgroup 0 also resets this launch's tickets and readiness counters
     // (nothing reads them before the second barrier) and the next launch's member counts.
     if (blockIdx.x == 0) {
+        // (written through the L2 like everything that crosses workgroups: the others hit these
+        // words with device-scope atomics)
         if (tid < uint32_t(kXcds)) {
-            sched[kSchedTicket + tid * kSchedLine] = 0u;
-            sched[kSchedMembers + (((seq + 1u) & 1u) * kXcds + tid) * kSchedLine] = 0u;
+            atomic_store_relaxed(sched + kSchedTicket + tid * kSchedLine, 0u);
+            atomic_store_relaxed(sched + kSchedMembers + (((seq + 1u) & 1u) * kXcds + tid) * kSchedLine, 0u);
         }
-        for (uint32_t i = tid; i < p.E * mt_max; i += kThreads) sched[kSchedReady + i] = 0u;
+        for (uint32_t i = tid; i < p.E * mt_max; i += kThreads) atomic_store_relaxed(sched + kSchedReady + i, 0u);
     }
     bool gate_done = false;
     if constexpr (sizeof(T) == 2 && (NG == 0 || NG >= 8)) {   // more than 64 experts
@@ -746,7 +748,7 @@ __global__ __launch_bounds__((TileShape<T, V>::kThreads), (TileShape<T, V>::kPer
     uint32_t q_off = 0;   // queues already found empty, starting from this workgroup's own XCD
     uint32_t q_dead = 0;  // bit q: queue q was seen exhausted
     bool q_scanned = false;
-    const Readiness rd{sched, mt_max, tn_up, p.wait_ticks, use_static};
+    const Readiness rd{sched, mt_max, tn_up, p.wait_ticks};
     auto decode = [&](Task& t, uint32_t q, uint32_t ticket) {
         uint32_t sg = s_qseg[q];
         const uint32_t sg_end = s_qseg[q + 1];

@@ -462,6 +462,41 @@ def test_fine_e256_top8_full_size(mode):
     assert v["expert_count"].astype(np.int64).sum() == c.S * c.k
 
 
+@pytest.mark.parametrize("name,schedule", [("headline_e64_zipf", ka.SCHEDULE_STATIC), ("headline_e64_zipf", ka.SCHEDULE_DYNAMIC),
+                                           ("balanced_e16", ka.SCHEDULE_AUTO), ("fine_e256_top8", ka.SCHEDULE_AUTO)],
+                         ids=["headline-static", "headline-dynamic", "balanced_e16", "fine_e256_top8"])
+def test_full_size_batches_alternate_in_one_context(name, schedule):
+    """Inside the persistent launch the routing tables, the slot tables, h1 and y pass between
+    workgroups on different XCDs, whose L2 caches are not coherent: a reader that got a line as an
+    earlier launch left it would compute with the other batch's data. Two full-size batches with
+    different routing alternate through one context, every CU busy; each output must equal, bit for
+    bit, what the same batch gives launch by launch (phased mode, where kernel boundaries do the
+    synchronisation)."""
+    w = synth.WORKLOADS[name]
+    c = moe_ref.cfg_from_keys(w.config)
+    batches = [synth.make_inputs(w, seed=seed, device="cuda")[0] for seed in (0, 1)]
+    refs = []
+    for iP in batches:
+        _, oP, v = run_gpu(w.config, iP, (ka.MODE_PHASED, ka.SCHEDULE_AUTO))
+        refs.append((_out_to_np(c, oP), v["topk_slot"].copy(), v["slot_token"].copy()))
+        del oP
+    assert not np.array_equal(refs[0][1], refs[1][1])
+    d = ka.initialize(w.config)
+    try:
+        _apply((ka.MODE_FUSED, schedule))
+        oP = synth.alloc_outputs(d)
+        for step, b in enumerate((0, 1, 1, 0, 1, 0)):
+            oP.fill_(float("nan"))
+            torch.cuda.synchronize()
+            ka.moe.forward_host(batches[b], oP)
+            ka.moe.stream_synchronize()
+            v = ka.moe.debug_views(d)
+            np.testing.assert_array_equal(v["topk_slot"], refs[b][1], err_msg=f"step {step}")
+            np.testing.assert_array_equal(_out_to_np(c, oP), refs[b][0], err_msg=f"step {step}")
+    finally:
+        ka.finalize()
+
+
 # ------------------------------------------------------------------ training mode
 @pytest.mark.parametrize("E,k,S", [(16, 2, 1024), (64, 2, 2048), (130, 8, 512), (384, 4, 512)])
 def test_training_mode_gate_loss(E, k, S):
