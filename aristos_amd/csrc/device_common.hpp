@@ -87,6 +87,36 @@ __device__ __forceinline__ f32x4 mma16_step(u32x4 a, u32x4 b, f32x4 acc, float) 
     return acc;
 }
 
+// The value another lane of the same row of 16 lanes holds, by the lane selects of the vector ALU
+// (no trip through the LDS crossbar as a general shuffle takes). STEP 0: lane ^ 1, 1: lane ^ 2,
+// 2: lane ^ 7, 3: lane ^ 15. Steps 0..3 in this order are an all-reduce over the 16 lanes for any
+// operation whose result does not depend on the order of its two operands: after steps 0 and 1 the
+// four lanes of a quad agree, so the mirrored lane of step 2 (in the other quad of the same eight)
+// holds what lane ^ 4 holds, and likewise lane ^ 15 what lane ^ 8 holds in step 3.
+template <int STEP>
+__device__ __forceinline__ uint32_t row16_peer(uint32_t v) {
+    static_assert(STEP >= 0 && STEP < 4);
+    constexpr int kCtrl = STEP == 0 ? 0xB1      // quad_perm [1, 0, 3, 2]
+                        : STEP == 1 ? 0x4E      // quad_perm [2, 3, 0, 1]
+                        : STEP == 2 ? 0x141     // row_half_mirror
+                                    : 0x140;    // row_mirror
+    return uint32_t(__builtin_amdgcn_update_dpp(0, int(v), kCtrl, 0xF, 0xF, false));
+}
+template <int STEP>
+__device__ __forceinline__ float row16_peer(float v) {
+    return __builtin_bit_cast(float, row16_peer<STEP>(__builtin_bit_cast(uint32_t, v)));
+}
+// op(a, b) == op(b, a) bit for bit (max, +): every lane of the row ends with the same value, combined
+// in the order of a xor butterfly over 1, 2, 4, 8.
+template <typename Op>
+__device__ __forceinline__ float row16_allreduce(float v, Op op) {
+    v = op(v, row16_peer<0>(v));
+    v = op(v, row16_peer<1>(v));
+    v = op(v, row16_peer<2>(v));
+    v = op(v, row16_peer<3>(v));
+    return v;
+}
+
 // Waits until at most N of this wavefront's vector-memory operations (loads and stores alike) are
 // outstanding.
 template <int N>

@@ -237,28 +237,54 @@ __device__ __forceinline__ void gate_unit(const LayerParams& p, uint32_t unit, f
         for (int g = 0; g < NG; ++g) acc[b][g] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     // logits^T: experts are the matrix-core rows, tokens its columns (gate.cuh:526-534). The loads
-    // of U steps are issued together before their matrix instructions: the activation rows stream
-    // from HBM once and this is what keeps enough of them in flight.
+    // of U steps are in flight together: the activation rows stream from HBM once and this is what
+    // keeps enough of them in flight. They are issued in halves of U / 2 steps, and a half is
+    // requested again (for U steps further on) as soon as its matrix instructions have read it, so
+    // the memory pipeline never runs empty between one batch and the next (worth 0.5 us of 12.5 per
+    // workgroup at the 64-expert shape with a hidden size of 2048: the loop runs at what a CU gets
+    // of the memory system while all CUs stream, about 32 GB/s).
     constexpr int U = NG <= 2 ? 8 : (NG <= 4 ? 4 : (NG <= 8 ? 2 : 1));
+    constexpr int UH = U >= 2 ? U / 2 : 1;
     uint32_t s = s0;
-    for (; s + U <= s1; s += U) {
+    if constexpr (U >= 2) {
         u32x4 xb[U][TB], wa[U][NG];
+        auto issue = [&](auto first_slot, uint32_t s_first) {
+            constexpr int u0 = decltype(first_slot)::value;
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            const uint32_t off = (s + u) * kStepK;
+            for (int u = 0; u < UH; ++u) {
+                const uint32_t off = (s_first + u) * kStepK;
 #pragma unroll
-            for (int b = 0; b < TB; ++b) xb[u][b] = load16(xrow[b] + off);
+                for (int b = 0; b < TB; ++b) xb[u0 + u][b] = load16(xrow[b] + off);
 #pragma unroll
-            for (int g = 0; g < NG; ++g) wa[u][g] = load16(wrow + size_t(g) * 16 * H + off);
+                for (int g = 0; g < NG; ++g) wa[u0 + u][g] = load16(wrow + size_t(g) * 16 * H + off);
+            }
+            __builtin_amdgcn_sched_barrier(0);   // the loads stay where they are written
+        };
+        auto consume = [&](auto first_slot) {
+            constexpr int u0 = decltype(first_slot)::value;
+#pragma unroll
+            for (int u = 0; u < UH; ++u)
+#pragma unroll
+                for (int g = 0; g < NG; ++g)
+#pragma unroll
+                    for (int b = 0; b < TB; ++b) acc[b][g] = mma16_step(wa[u0 + u][g], xb[u0 + u][b], acc[b][g], T{});
+            __builtin_amdgcn_sched_barrier(0);
+        };
+        constexpr std::integral_constant<int, 0> lower{};
+        constexpr std::integral_constant<int, UH> upper{};
+        if (s + U <= s1) {
+            issue(lower, s);
+            issue(upper, s + UH);
+            for (; s + 2 * U <= s1; s += U) {
+                consume(lower);
+                issue(lower, s + U);
+                consume(upper);
+                issue(upper, s + U + UH);
+            }
+            consume(lower);
+            consume(upper);
+            s += U;
         }
-        // every load above is issued before the first matrix instruction waits for one of them
-        __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int u = 0; u < U; ++u)
-#pragma unroll
-            for (int g = 0; g < NG; ++g)
-#pragma unroll
-                for (int b = 0; b < TB; ++b) acc[b][g] = mma16_step(wa[u][g], xb[u][b], acc[b][g], T{});
     }
     for (; s < s1; ++s) {
         const uint32_t off = s * kStepK;
@@ -648,15 +674,13 @@ __device__ __forceinline__ void gate_group_finish(const LayerParams& p, uint32_t
                 m = fmaxf(m, acc[j][v]);
             }
         }
-#pragma unroll
-        for (int off = 1; off <= 8; off <<= 1) m = fmaxf(m, __shfl_xor(m, off));
+        m = row16_allreduce(m, [](float a, float b) { return fmaxf(a, b); });
         float d = 0.f;
 #pragma unroll
         for (int j = 0; j < NL; ++j)
 #pragma unroll
             for (int v = 0; v < 4; ++v) d += __expf(acc[j][v] - m);
-#pragma unroll
-        for (int off = 1; off <= 8; off <<= 1) d += __shfl_xor(d, off);
+        d = row16_allreduce(d, [](float a, float b) { return a + b; });
         const float inv_d = 1.0f / d;
         auto prob = [&](float logit) { return __expf(logit - m) * inv_d; };
         // gateOut[t, e] = Element(p) (gate.cuh:590-605); padded columns are zero
@@ -695,15 +719,17 @@ __device__ __forceinline__ void gate_group_finish(const LayerParams& p, uint32_t
                         best = w[j][v];
                         bi = 64 * j + 4 * sub + v;
                     }
-#pragma unroll
-            for (int off = 1; off <= 8; off <<= 1) {
-                const float ob = __shfl_xor(best, off);
-                const uint32_t oi = __shfl_xor(bi, off);
+            // (the rule is symmetric in the two candidates, so the lanes of a pair agree after a step)
+            auto better = [&](float ob, uint32_t oi) {
                 if (oi != kNone && (bi == kNone || ob > best || (ob == best && oi < bi))) {
                     best = ob;
                     bi = oi;
                 }
-            }
+            };
+            { const float ob = row16_peer<0>(best); const uint32_t oi = row16_peer<0>(bi); better(ob, oi); }
+            { const float ob = row16_peer<1>(best); const uint32_t oi = row16_peer<1>(bi); better(ob, oi); }
+            { const float ob = row16_peer<2>(best); const uint32_t oi = row16_peer<2>(bi); better(ob, oi); }
+            { const float ob = row16_peer<3>(best); const uint32_t oi = row16_peer<3>(bi); better(ob, oi); }
             // every lane of the token knows the winner and its logit
             const float pv = bi != kNone ? prob(best) : 0.f;
             den += pv;   // mCw, accumulated in selection order (gate.cuh:669)
