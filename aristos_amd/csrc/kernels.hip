@@ -630,19 +630,7 @@ __global__ __launch_bounds__((TileShape<T, V>::kThreads), (TileShape<T, V>::kPer
     grid_barrier(sched, p.wait_ticks, 0, seq, nwg);
     if (tid == 0) stamp[2] = wall_clock64();
 
-    // ---- phase 1: slots in token order
-    {
-        uint32_t* base = reinterpret_cast<uint32_t*>(smem) + wave * p.E;
-        // wavefront w of workgroup b takes tile b + w * nwg: the tiles spread over all CUs
-        for (uint32_t t0 = blockIdx.x; t0 < p.n_gate_tiles; t0 += nwg * kWaves)
-            slot_tile(p, t0 + wave * nwg, t0 + wave * nwg < p.n_gate_tiles, base);
-        uint32_t* other = p.super_count + size_t((p.epoch & 1u) ^ 1u) * p.n_super * p.E;
-        for (uint32_t i = blockIdx.x * kThreads + tid; i < p.n_super * p.E; i += nwg * kThreads) other[i] = 0u;
-    }
-    if (tid == 0) stamp[3] = wall_clock64();
-
-    // ---- phase 2: expert tiles from the per-XCD queues (by ticket, or by stride in the static schedule)
-    // LDS map: row blocks per expert | queue starts, totals, task | segments | GEMM tile
+    // LDS map of the expert phase: row blocks per expert | queue starts, totals, task | segments | GEMM tile
     uint32_t* s_rows = reinterpret_cast<uint32_t*>(smem);                       // [E] rows kept
     uint16_t* s_mt = reinterpret_cast<uint16_t*>(smem + 4 * lds_experts(p.E));  // [E] row blocks
     uint32_t* s_qseg = reinterpret_cast<uint32_t*>(smem + lds_queue_offset(p.E));   // [9] first segment of each queue
@@ -658,25 +646,45 @@ __global__ __launch_bounds__((TileShape<T, V>::kThreads), (TileShape<T, V>::kPer
     char* s_gemm = smem + fused_lds_header(p.E);
     const uint32_t tn_up = ceil_div_u32(p.I, BN), tn_down = ceil_div_u32(p.H, BN);
 
-    // The queues of the expert phase are set up while this workgroup waits for the others to finish
-    // the slot phase: what the set-up reads (the routed counts the gate accumulated, the workgroups
-    // per XCD) has been complete since the first barrier.
-    const uint32_t members = nwg / kXcds;
-    bool use_static = false;
-    grid_barrier(sched, p.wait_ticks, 1, seq, nwg, [&] {
-        // how many workgroups every XCD holds: asked for first, so that the answers travel together
-        // with the routed counts below
-        uint32_t seen[kXcds] = {};
-        if (tid == 0)
+    // ---- phase 1: slots in token order
+    {
+        // Rows and row blocks per expert and the workgroups per XCD, for the queues of the expert
+        // phase: what this reads (the routed counts the gate accumulated, the member counts) has been
+        // complete since the first barrier, so its trips to memory ride along with the slot tiles. The threads at the top of the workgroup take it:
+        // the slot tiles go to the wavefronts at the bottom.
+        if (tid == kThreads - 1) {
+            // the static schedule needs every XCD to hold the same number of workgroups
+            uint32_t seen[kXcds];   // all eight asked for before the first answer is looked at
             for (uint32_t j = 0; j < kXcds; ++j) seen[j] = atomic_load_relaxed(members_now + j * kSchedLine);
-        for (uint32_t e = tid; e < p.E; e += kThreads) {
+            bool even = nwg % kXcds == 0;
+            for (uint32_t j = 0; j < kXcds; ++j) even = even && seen[j] == nwg / kXcds;
+            s_static[5] = even;
+        }
+        for (uint32_t e = kThreads - 1 - tid; e < p.E; e += kThreads) {
             const uint32_t routed = routed_count(p, e);
             const uint32_t cap = p.EC < p.cap_rows ? p.EC : p.cap_rows;
             const uint32_t rows = routed < cap ? routed : cap;   // consumers clamp the routed count to the capacity (packet.cuh:85,112-113)
             s_rows[e] = rows;
             s_mt[e] = uint16_t(ceil_div_u32(rows, BM));
         }
-        __syncthreads();
+        // (the slot tiles' scratch sits in the GEMM tile's memory, clear of the words above)
+        uint32_t* base = reinterpret_cast<uint32_t*>(s_gemm) + wave * p.E;
+        // wavefront w of workgroup b takes tile b + w * nwg: the tiles spread over all CUs
+        for (uint32_t t0 = blockIdx.x; t0 < p.n_gate_tiles; t0 += nwg * kWaves)
+            slot_tile(p, t0 + wave * nwg, t0 + wave * nwg < p.n_gate_tiles, base);
+        uint32_t* other = p.super_count + size_t((p.epoch & 1u) ^ 1u) * p.n_super * p.E;
+        for (uint32_t i = blockIdx.x * kThreads + tid; i < p.n_super * p.E; i += nwg * kThreads) other[i] = 0u;
+    }
+    if (tid == 0) stamp[3] = wall_clock64();
+
+    // ---- phase 2: expert tiles from the per-XCD queues (by ticket, or by stride in the static schedule)
+    // The queues of the expert phase are set up while this workgroup waits for the others to finish
+    // the slot phase: what the set-up reads (the rows per expert worked out above, the workgroups
+    // per XCD) has been complete since the first barrier.
+    const uint32_t members = nwg / kXcds;
+    bool use_static = false;
+    grid_barrier(sched, p.wait_ticks, 1, seq, nwg, [&] {
+        __syncthreads();   // the rows per expert are in place
         // Static or dynamic schedule: every workgroup decides alike, from the same counters.
         // Static: each XCD's workgroups stride through their queue (all its up tiles, then all its
         // down tiles) by their rank: no tickets, no stealing, nothing written back from the L2 per
@@ -690,11 +698,8 @@ __global__ __launch_bounds__((TileShape<T, V>::kThreads), (TileShape<T, V>::kPer
             s_qtot[tid] = blocks;
         }
         if (tid == 0) {
-            bool even = nwg % kXcds == 0;
-            for (uint32_t j = 0; j < kXcds; ++j) even = even && seen[j] == members;
             s_static[1] = my_rank;
             s_static[3] = my_rank;
-            s_static[5] = even;
         }
         __syncthreads();
         {
@@ -811,7 +816,8 @@ template <typename T, int NG, int V>
 size_t fused_smem_bytes(uint32_t E) {
     size_t need = fused_lds_header(E) + gemm_smem_bytes<T, V>();
     const size_t gate = gate_smem_floats<NG>(TileShape<T>::kThreads / kWave) * sizeof(float);
-    const size_t slots = (TileShape<T>::kThreads / kWave) * size_t(E) * sizeof(uint32_t);
+    // the slot tiles' scratch sits behind the header of the expert phase
+    const size_t slots = fused_lds_header(E) + (TileShape<T>::kThreads / kWave) * size_t(E) * sizeof(uint32_t);
     if (gate > need) need = gate;
     if (slots > need) need = slots;
     if constexpr (sizeof(T) == 2) {
