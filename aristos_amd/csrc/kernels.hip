@@ -591,8 +591,8 @@ __global__ __launch_bounds__((TileShape<T, V>::kThreads), (TileShape<T, V>::kPer
     unsigned long long* stamp = p.stamps + size_t(blockIdx.x) * kStampWords;
     if (tid == 0) stamp[0] = wall_clock64();
 
-    // The XCD this workgroup really runs on (hardware register XCC_ID): expert e's tiles are queued
-    // on XCD e % 8, so that its weights, its gathered rows and the h1 rows handed from its
+    // The XCD this workgroup really runs on (hardware register XCC_ID): all tiles of an expert are
+    // queued on one XCD, so that its weights, its gathered rows and the h1 rows handed from its
     // up-projection to its down-projection all live in one L2. Every workgroup also takes a rank
     // among the workgroups of its XCD, which the static schedule strides by.
     const uint32_t xcd = __builtin_amdgcn_s_getreg((3 << 11) | 20) & (kXcds - 1);
@@ -646,6 +646,47 @@ __global__ __launch_bounds__((TileShape<T, V>::kThreads), (TileShape<T, V>::kPer
     char* s_gemm = smem + fused_lds_header(p.E);
     const uint32_t tn_up = ceil_div_u32(p.I, BN), tn_down = ceil_div_u32(p.H, BN);
 
+    // Which queue (XCD) an expert goes to. With more than 64 experts they are dealt out in descending
+    // order of their rows, forwards and backwards in turn (queues 0..7, then 7..0, ...), so that every
+    // queue holds about the same number of rows as well as of experts: an expert's tiles cost the more
+    // the more rows it really holds (padding rows repeat one address). 256-expert top-8 shape: 2.92
+    // against 2.96 ms per forward with the placement by index. Every workgroup computes the same
+    // placement from the same counts.
+    //   s_place[q * per_q + i]: the i-th expert of queue q.
+    const uint32_t per_q = ceil_div_u32(p.E, kXcds);
+    uint16_t* s_place = reinterpret_cast<uint16_t*>(s_gemm + size_t(kWaves) * p.E * sizeof(uint32_t));
+    auto place = [&](uint32_t e) {
+        const uint32_t mine = s_rows[e];
+        uint32_t rank = 0;   // experts with more rows, or as many and a lower index
+        // (sixteen counts per trip to LDS; the array is padded to a multiple of 64 words)
+        for (uint32_t o0 = 0; o0 < p.E; o0 += 16) {
+            u32x4 v[4];
+#pragma unroll
+            for (uint32_t j = 0; j < 4; ++j) v[j] = *reinterpret_cast<const u32x4*>(s_rows + o0 + 4 * j);
+#pragma unroll
+            for (uint32_t j = 0; j < 16; ++j) {
+                const uint32_t o = o0 + j, other = v[j / 4][j % 4];
+                rank += uint32_t(o < p.E && (other > mine || (other == mine && o < e)));
+            }
+        }
+        const uint32_t round = rank / kXcds, pos = rank % kXcds;
+        s_place[((round & 1u) ? kXcds - 1 - pos : pos) * per_q + round] = uint16_t(e);
+    };
+    // Up to 64 experts keep the placement by index (expert e in queue e mod 8, nothing to look up):
+    // with at most eight experts to a queue the ranking costs the slot phase more than even rows bring.
+    const bool by_index = p.E <= uint32_t(kWave);
+    auto expert_at = [&](uint32_t q, uint32_t i) -> uint32_t {
+        if (by_index) return q + kXcds * i;
+        return s_place[q * per_q + i];
+    };
+    // experts in queue q: the full rounds, and the last, partial one from whichever end it starts at
+    // (always from queue 0 with the placement by index)
+    auto experts_in = [&](uint32_t q) {
+        const uint32_t full = p.E / kXcds, rest = p.E % kXcds;
+        const bool backwards = !by_index && (full & 1u);
+        return full + uint32_t(rest != 0 && (backwards ? q >= kXcds - rest : q < rest));
+    };
+
     // ---- phase 1: slots in token order
     {
         // Rows and row blocks per expert and the workgroups per XCD, for the queues of the expert
@@ -672,6 +713,10 @@ __global__ __launch_bounds__((TileShape<T, V>::kThreads), (TileShape<T, V>::kPer
         // wavefront w of workgroup b takes tile b + w * nwg: the tiles spread over all CUs
         for (uint32_t t0 = blockIdx.x; t0 < p.n_gate_tiles; t0 += nwg * kWaves)
             slot_tile(p, t0 + wave * nwg, t0 + wave * nwg < p.n_gate_tiles, base);
+        if (!by_index) {
+            __syncthreads();   // the counts of all wavefronts
+            for (uint32_t e = tid; e < p.E; e += kThreads) place(e);
+        }
         uint32_t* other = p.super_count + size_t((p.epoch & 1u) ^ 1u) * p.n_super * p.E;
         for (uint32_t i = blockIdx.x * kThreads + tid; i < p.n_super * p.E; i += nwg * kThreads) other[i] = 0u;
     }
@@ -684,17 +729,17 @@ __global__ __launch_bounds__((TileShape<T, V>::kThreads), (TileShape<T, V>::kPer
     const uint32_t members = nwg / kXcds;
     bool use_static = false;
     grid_barrier(sched, p.wait_ticks, 1, seq, nwg, [&] {
-        __syncthreads();   // the rows per expert are in place
+        __syncthreads();   // the rows per expert and their queues are in place
         // Static or dynamic schedule: every workgroup decides alike, from the same counters.
         // Static: each XCD's workgroups stride through their queue (all its up tiles, then all its
         // down tiles) by their rank: no tickets, no stealing, nothing written back from the L2 per
         // tile. It needs every XCD to hold the same number of workgroups, and it pays only when no
         // queue would keep its XCD busy for longer than freely handed-out tiles keep the grid busy.
         // Thread q sets up queue q; its segments start at a fixed place, two per expert of the queue.
-        const uint32_t my_nq = tid < p.E && tid < uint32_t(kXcds) ? (p.E - tid + kXcds - 1) / kXcds : 0u;   // experts q, q+8, ...
+        const uint32_t my_nq = tid < uint32_t(kXcds) ? experts_in(tid) : 0u;
         if (tid < uint32_t(kXcds)) {
             uint32_t blocks = 0;
-            for (uint32_t i = 0; i < my_nq; ++i) blocks += s_mt[tid + kXcds * i];
+            for (uint32_t i = 0; i < my_nq; ++i) blocks += s_mt[expert_at(tid, i)];
             s_qtot[tid] = blocks;
         }
         if (tid == 0) {
@@ -721,7 +766,8 @@ __global__ __launch_bounds__((TileShape<T, V>::kThreads), (TileShape<T, V>::kPer
         __syncthreads();   // the row-block sums above shared s_qtot with the ticket totals below
         if (tid < uint32_t(kXcds)) {
             const uint32_t q = tid, nq = my_nq;
-            const uint32_t first = 2 * (q * (p.E / kXcds) + (q < p.E % kXcds ? q : p.E % kXcds));
+            uint32_t first = 0;   // two segments per expert of the queues before this one
+            for (uint32_t j = 0; j < q; ++j) first += 2 * experts_in(j);
             uint32_t nseg = first;
             s_qseg[q] = first;
             if (q == kXcds - 1) s_qseg[kXcds] = 2 * p.E;
@@ -732,13 +778,13 @@ __global__ __launch_bounds__((TileShape<T, V>::kThreads), (TileShape<T, V>::kPer
             // up tiles it depends on have normally been stored.
             for (uint32_t i = 0; i < nq + lag; ++i) {
                 if (i < nq) {
-                    const uint32_t e = q + kXcds * i;
+                    const uint32_t e = expert_at(q, i);
                     s_seg[nseg++] = Segment{uint16_t(e), 0, 0, ticket};
                     ticket += uint32_t(s_mt[e]) * tn_up;
                     ups += uint32_t(s_mt[e]) * tn_up;
                 }
                 if (i >= lag && i - lag < nq) {
-                    const uint32_t e = q + kXcds * (i - lag);
+                    const uint32_t e = expert_at(q, i - lag);
                     s_seg[nseg++] = Segment{uint16_t(e), 1, 0, ticket};
                     ticket += uint32_t(s_mt[e]) * tn_down;
                 }
@@ -817,7 +863,8 @@ size_t fused_smem_bytes(uint32_t E) {
     size_t need = fused_lds_header(E) + gemm_smem_bytes<T, V>();
     const size_t gate = gate_smem_floats<NG>(TileShape<T>::kThreads / kWave) * sizeof(float);
     // the slot tiles' scratch sits behind the header of the expert phase
-    const size_t slots = fused_lds_header(E) + (TileShape<T>::kThreads / kWave) * size_t(E) * sizeof(uint32_t);
+    const size_t slots = fused_lds_header(E) + (TileShape<T>::kThreads / kWave) * size_t(E) * sizeof(uint32_t) +
+                         kXcds * size_t(ceil_div_u32(E, kXcds)) * sizeof(uint16_t);   // and the experts of each queue behind it
     if (gate > need) need = gate;
     if (slots > need) need = slots;
     if constexpr (sizeof(T) == 2) {
