@@ -290,6 +290,36 @@ struct Gemm16 {
         const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
         const int wm = wave / WAVES_N, wn = wave % WAVES_N;
         const int fr_row = lane & 31, fr_half = lane >> 5;
+        if (rows_absent(t, __builtin_amdgcn_readfirstlane(wave) / WAVES_N)) {   // (a scalar condition: the branch holds barriers)
+            // None of this wavefront's rows exist (an expert with few rows): it brings its share of
+            // every slice into LDS at the same points of the same sequence of barriers as the others,
+            // and leaves the fragment reads and the matrix instructions out.
+            if constexpr (AHEAD2) {
+                asm volatile("s_barrier" ::: "memory");
+                if (t.k_tiles > 1) issue_slice(t, smem, 1);
+                for (uint32_t kt = 0; kt < t.k_tiles; ++kt) {
+                    if (kt + 1 < t.k_tiles) wait_vmcnt<kLoadsPerSlice>();
+                    else wait_vmcnt<0>();
+                    asm volatile("s_barrier" ::: "memory");
+                    if (kt == 0) after_first_barrier();
+                    if (kt + 2 < t.k_tiles) {
+                        asm volatile("s_barrier" ::: "memory");
+                        issue_slice(t, smem, kt + 2);
+                    }
+                }
+            } else {
+                for (uint32_t kt = 0; kt < t.k_tiles; ++kt) {
+                    const uint32_t later = t.k_tiles - 1 - kt;
+                    if (STAGES >= 4 && later >= 2) wait_vmcnt<(STAGES >= 4 ? 2 : 0) * kLoadsPerSlice>();
+                    else if (STAGES >= 3 && later >= 1) wait_vmcnt<kLoadsPerSlice>();
+                    else wait_vmcnt<0>();
+                    asm volatile("s_barrier" ::: "memory");
+                    if (kt == 0) after_first_barrier();
+                    if (kt + (STAGES - 1) < t.k_tiles) issue_slice(t, smem, kt + STAGES - 1);
+                }
+            }
+            return;
+        }
 #pragma unroll
         for (int ni = 0; ni < TN; ++ni)
 #pragma unroll
@@ -426,6 +456,17 @@ struct Gemm16 {
         }
     }
 
+    // Whether none of the rows of the wavefronts in row wm of the wavefront grid exist in this tile
+    // (the same for all lanes of a wavefront), for the configurations that treat such wavefronts
+    // apart: the one with the loads two slices ahead, which runs where experts hold few rows and
+    // the loads bound the tile (64-expert shape with skewed routing: 301 against 304 us per forward);
+    // where the matrix work bounds it the extra branch costs more than the few such tiles bring
+    // (8-expert shape with hidden size 4096: 3.57 against 3.53 ms).
+    static __device__ __forceinline__ bool rows_absent(const Tile& t, int wm) {
+        if constexpr (AHEAD2) return uint32_t(wm * WM) >= t.m_valid;
+        else return false;
+    }
+
     // The stage the tile's last K slice was read from (free once every wavefront has left mainloop()).
     static __device__ __forceinline__ int last_stage(const Tile& t) { return (t.stage0 + t.k_tiles - 1) % STAGES; }
     // The stage the next tile's first slice must go to.
@@ -465,6 +506,7 @@ struct Gemm16 {
 
     // Epilogue. Every wavefront must have left mainloop().
     static __device__ __forceinline__ void finish(const Tile& t, Acc& acc, char* smem) {
+        if (rows_absent(t, __builtin_amdgcn_readfirstlane(int(local_tid() >> 6)) / WAVES_N)) return;   // nothing of this wavefront's is stored
         const TileOut out{t.c_base, t.ldc, t.m_valid, t.n_valid, t.act};
         epilogue16<E, WM, WN, WAVES_N>(out, acc, smem + last_stage(t) * kStage, smem + kBiasOffset + t.bias_slot * kBiasBytes);
     }
