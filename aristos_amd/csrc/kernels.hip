@@ -31,23 +31,27 @@ namespace {
 
 constexpr int kXcds = 8;
 // Expert GEMM configuration of the bf16 / fp16 path: 256 x 256 tile (an expert's whole capacity of
-// 256 rows at the headline shape, so its weights stream from HBM exactly once), 2 x 4 wavefronts of
-// 128 x 64 (two per SIMD), K slices of 64 (whole 128-byte lines of every row) through two 64 KB
+// 256 rows at the headline shape, so its weights stream from HBM exactly once), 4 x 2 wavefronts of
+// 64 x 128 (two per SIMD), K slices of 64 (whole 128-byte lines of every row) through two 64 KB
 // stages, loads two slices ahead.
 // (Measured against it on MI355X, none faster: K slices of 32 through four stages, 2 x 2 wavefronts
 // of 128 x 128 with the accumulators in AGPRs, weight slices of 64 through three slots with
-// activation half slices of 32 through three, the 128 x 256 tile of variant 1.)
+// activation half slices of 32 through three, the 128 x 256 tile of variant 1. 2 x 4 wavefronts
+// of 128 x 64: 305.0 against 299.8 us per forward at the headline shape, 158.3 against 155.7 at
+// the 16-expert shape, whose tiles are all full; with four rows of wavefronts those whose rows do
+// not exist in a tile also come in steps of 64 rows.)
 // Variant 1, for layers whose experts hold at most 128 rows (many small experts): a 128 x 256 tile
 // wastes no matrix work and no activation loads on rows that do not exist, and its smaller stages
 // leave room for a third one (measured on the 256-expert top-8 shape: 3.7 ms against 4.6 ms).
 // Variant 2, for layers whose experts hold at least four row blocks (few large experts: every
 // weight tile is shared by several workgroups through L2, loads return quickly and the matrix work
-// dominates): the tile of variant 0 with the loads one slice ahead, issued during the first K step.
+// dominates): the tile of variant 0 on 2 x 4 wavefronts of 128 x 64 (3.53 against 3.57 ms with 4 x 2
+// at the 8-expert shape with hidden size 4096), the loads one slice ahead, issued during the first K step.
 // Variants 0 and 1 load their weight rows non-temporally (headline 378 against 390 us per forward,
 // the 16-expert shape 192 against 196, the 256-expert shape 3.43 against 3.48 ms); variant 2, whose
 // weight tiles are shared by eight workgroups and more, does not (4.06 against 4.01 ms with it).
 template <typename E, int V>
-using GemmCfg = std::conditional_t<V == 0, Gemm16<E, 256, 256, 2, 4, 64, 2, true, true>,
+using GemmCfg = std::conditional_t<V == 0, Gemm16<E, 256, 256, 4, 2, 64, 2, true, true>,
                 std::conditional_t<V == 1, Gemm16<E, 128, 256, 2, 4, 64, 3, true, false>, Gemm16<E, 256, 256, 2, 4, 64, 2, false, false>>>;
 constexpr int kBN = 256;
 constexpr int kGemmThreads = GemmCfg<bf16_t, 0>::kThreads;
