@@ -247,6 +247,26 @@ def test_identity_experts_return_input(mode):
 
 # ------------------------------------------------------------------ back-to-back launches
 @pytest.mark.parametrize("mode", MODES, ids=MODE_IDS)
+def test_experts_that_fill_a_tile_to_every_quarter(mode):
+    """256-row tiles (the variant for experts of 129 to 1023 rows) whose experts hold 12, 62, 81, 147, 220
+    and 256 + 64 rows: the wavefronts of a tile own 64 rows each, and those whose rows do not exist leave
+    the arithmetic of the tile out. A constant input feature times a per-expert gate weight skews the
+    routing; the two hottest experts overflow their capacity of 512."""
+    keys = _keys(1024, 128, 256, 8, 2, cf=2.0)
+    c = moe_ref.cfg_from_keys(keys)
+    assert c.EC == 512
+    x, wg, w_up, w_down, *_ = random_layer(c, seed=77, w_std=0.08)
+    x[:, 0] = 4.0
+    wg[:, 0] = np.array([1.2, 0.9, 0.6, 0.3, 0.1, -0.1, -0.4, -0.9], np.float32) * 0.3
+    iP = pack_inputs(c, x, wg, w_up, w_down)
+    d, v, moe_out, err = check_against_oracle(c, keys, iP, mode)
+    kept = np.minimum(v["expert_count"].astype(np.int64), c.EC) % 256
+    quarters = {int((r - 1) // 64) for r in kept if r}
+    assert quarters == {0, 1, 2, 3}, sorted(kept)
+    assert (v["topk_slot"] < 0).sum() > 0
+
+
+@pytest.mark.parametrize("mode", MODES, ids=MODE_IDS)
 def test_back_to_back_launches_need_no_host_reset(mode):
     """The reference resets its state inside the kernel (moe.cuh:31-70) so launches can follow each
     other; here the same must hold for counters and the double-buffered histograms. Five launches,
