@@ -55,6 +55,10 @@ SYMBOLS = {
     "kleos_moe_forward": (C.c_int, [C.c_void_p, C.c_void_p]),
     "kleos_moe_forward_bench": (C.c_int, [C.c_void_p, C.c_void_p, C.c_uint32, C.c_uint32, C.POINTER(C.c_float)]),
     "kleos_moe_forward_static_scratch": (C.c_int, [C.POINTER(KleosConfigStruct), C.c_void_p, C.c_void_p, C.c_void_p]),
+    "kleos_static_scratch_prepare": (C.c_int, [C.POINTER(KleosConfigStruct)]),
+    "kleos_static_scratch_status": (C.c_int, [C.c_void_p]),
+    "kleos_debug_static_scratch_expiry": (C.c_int, [C.c_ulonglong, C.c_uint32]),
+    "kleos_debug_map_hip_error": (C.c_int, [C.c_int]),
     "kleos_stream_synchronize": (C.c_int, []),
     "kleos_stream": (C.c_void_p, []),
     "kleos_set_mode": (C.c_int, [C.c_int]),

@@ -62,9 +62,10 @@ ArenaLayout layout_arena(const kleos_config_t& c, uint32_t n_tiles, uint32_t n_s
     auto take = [&](size_t bytes) { size_t o = off; off = align_up(off + bytes, 256); return o; };
     const size_t S = c.S, E = c.E, k = c.k, R = c.cap_rows;
     // counters first: they are the part cleared at initialisation
+    // (the scheduler words come first: the error word then sits at the same place in every layout)
     L.zero_begin = off;
-    L.super_count = take(2 * size_t(n_super) * E * 4);
     L.sched = take(sched_words(c.E, c.cap_rows) * 4);
+    L.super_count = take(2 * size_t(n_super) * E * 4);
     L.expert_count = take(E * 4);
     L.stamps = take(size_t(kMaxWorkgroups) * 16 * 8);
     L.gate_loss = take((2 * E + 1) * 4);
@@ -191,9 +192,22 @@ int enqueue_forward(Context& c, const void* iP, void* oP, hipEvent_t* ev) {
 // ---------------------------------------------------------------- the entry point that allocates nothing
 // Every library-owned array of a forward (routing tables, h1, y, scheduler counters, stamps) laid out
 // in a fixed array in device memory instead of an arena from hipMalloc. Every GPU the library runs
-// on holds its own copy of the array, at its own address, until the process ends.
+// on holds its own copy of the array, at its own address, until the process ends. The last 256
+// bytes of the array are not part of any layout: their first word is the sticky record of expired
+// waits that kleos_static_scratch_status reads.
 constexpr size_t kStaticScratchBytes = KLEOS_STATIC_SCRATCH_BYTES;
+constexpr size_t kStaticScratchTail = 256;
+constexpr size_t kStaticScratchUsable = kStaticScratchBytes - kStaticScratchTail;
 static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+// A plan of the persistent launch as a call found it, kept so that repeated calls with the same
+// layer make no runtime queries.
+struct CachedPlan {
+    bool used = false;
+    uint32_t dtype = 0, S = 0, H = 0, I = 0, E = 0, k = 0, EC = 0, cap_rows = 0, is_training = 0;
+    FusedPlan plan{};
+};
+constexpr int kCachedPlans = 16;
 
 // What a device needs once: the address of its copy of `scratch` (in host code the array's name is
 // only a handle for hipGetSymbolAddress, never a device address) and its compute-unit count.
@@ -202,13 +216,19 @@ struct DeviceSetup {
     char* scratch_ptr = nullptr;
     int num_cus = 0;
     bool gfx950 = false;
+    CachedPlan plans[kCachedPlans];
+    int next_plan = 0;
 };
 constexpr int kMaxDevices = 64;
 DeviceSetup g_devices[kMaxDevices];
 std::mutex g_devices_mutex;
+// Test hooks of the static-scratch path (kleos_debug_static_scratch_expiry): a tick budget for its
+// in-kernel waits and launch numbers to skip, which makes every barrier of its launches expire.
+unsigned long long g_static_wait_ticks = 0;
+uint32_t g_static_skip = 0;
 
 // Looks the current device up (first call per device) or returns what was found then.
-int device_setup(const DeviceSetup** out) {
+int device_setup(DeviceSetup** out) {
     int dev = -1;
     KLEOS_HIP(hipGetDevice(&dev));
     if (dev < 0 || dev >= kMaxDevices) return fail(KLEOS_EUNSUPPORTED, "device ordinal %d is beyond %d", dev, kMaxDevices);
@@ -229,8 +249,56 @@ int device_setup(const DeviceSetup** out) {
     return KLEOS_OK;
 }
 
-__global__ __launch_bounds__(256) void zero_words_kernel(uint32_t* words, size_t n) {
-    for (size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += size_t(gridDim.x) * blockDim.x) words[i] = 0u;
+// Clears the counter range of a layout. The thread that owns the error word first copies a set
+// word into the sticky record, so that an expired wait of the previous call stays on record until
+// kleos_static_scratch_status has reported it.
+__global__ __launch_bounds__(256) void zero_words_kernel(uint32_t* words, size_t n, size_t error_index, uint32_t* sticky) {
+    for (size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += size_t(gridDim.x) * blockDim.x) {
+        if (i == error_index && words[i] != 0u) *sticky = 1u;
+        words[i] = 0u;
+    }
+}
+
+// Everything a static-scratch call derives from its configuration before it touches the stream.
+struct StaticCall {
+    kleos_config_t cfg;
+    DeviceSetup* dev = nullptr;
+    LayerParams p{};
+    ArenaLayout L{};
+    FusedPlan plan{};
+};
+
+int prepare_static_call(const kleos_config_t* user_cfg, StaticCall& c) {
+    c.cfg = *user_cfg;
+    if (int rc = kleos_config_derive(&c.cfg)) return rc;
+    if (const char* why = unsupported_reason(c.cfg.E, c.cfg.k)) return fail(KLEOS_EUNSUPPORTED, "%s", why);
+    if (int rc = device_setup(&c.dev)) return rc;
+    if (!c.dev->gfx950) return fail(KLEOS_EUNSUPPORTED, "the current device is not gfx950: this library is built for MI355X only");
+    params_from_config(c.p, c.cfg);
+    c.p.gate_splits = gate_splits_for(c.cfg.S, c.cfg.H, c.cfg.E, c.cfg.PX, int(c.cfg.torch_dtype), c.dev->num_cus);
+    c.L = layout_arena(c.cfg, c.p.n_gate_tiles, c.p.n_super, c.p.gate_splits);
+    if (c.L.total > kStaticScratchUsable)
+        return fail(KLEOS_EUNSUPPORTED, "kleos_moe_forward_static_scratch: this configuration needs %zu bytes of library "
+                    "memory, the static scratch holds %zu; use kleos_initialize + kleos_moe_forward", c.L.total,
+                    kStaticScratchUsable);
+    if (c.L.sched != 0) return fail(KLEOS_EHIP, "static scratch: the scheduler words must open the layout");
+    params_from_arena(c.p, c.dev->scratch_ptr, c.L);
+    // the plan of this layer: looked up, or made once (function attributes, occupancy query) and kept
+    std::lock_guard<std::mutex> lock(g_devices_mutex);
+    const kleos_config_t& g = c.cfg;
+    for (CachedPlan& e : c.dev->plans)
+        if (e.used && e.dtype == g.torch_dtype && e.S == g.S && e.H == g.H && e.I == g.I && e.E == g.E && e.k == g.k &&
+            e.EC == g.EC && e.cap_rows == g.cap_rows && e.is_training == g.is_training) {
+            c.plan = e.plan;
+            return KLEOS_OK;
+        }
+    KLEOS_HIP(plan_fused(c.p, int(g.torch_dtype), c.dev->num_cus, &c.plan));
+    if (c.plan.nwg > kMaxWorkgroups) return fail(KLEOS_EUNSUPPORTED, "persistent grid of %u workgroups exceeds %u", c.plan.nwg, kMaxWorkgroups);
+    CachedPlan& e = c.dev->plans[c.dev->next_plan];
+    c.dev->next_plan = (c.dev->next_plan + 1) % kCachedPlans;
+    e.used = true; e.dtype = g.torch_dtype; e.S = g.S; e.H = g.H; e.I = g.I; e.E = g.E; e.k = g.k; e.EC = g.EC;
+    e.cap_rows = g.cap_rows; e.is_training = g.is_training; e.plan = c.plan;
+    return KLEOS_OK;
 }
 
 }  // namespace
@@ -238,39 +306,63 @@ __global__ __launch_bounds__(256) void zero_words_kernel(uint32_t* words, size_t
 
 using namespace kleos_amd;
 
+extern "C" int kleos_static_scratch_prepare(const kleos_config_t* user_cfg) {
+    if (!user_cfg) return fail(KLEOS_EINVAL, "kleos_static_scratch_prepare: null config");
+    StaticCall c;
+    return prepare_static_call(user_cfg, c);
+}
+
 extern "C" int kleos_moe_forward_static_scratch(const kleos_config_t* user_cfg, const void* iP, void* oP, void* stream) {
     if (!user_cfg) return fail(KLEOS_EINVAL, "kleos_moe_forward_static_scratch: null config");
     if (!iP || !oP) return fail(KLEOS_EINVAL, "kleos_moe_forward_static_scratch: null buffer");
     if ((reinterpret_cast<uintptr_t>(iP) | reinterpret_cast<uintptr_t>(oP)) & 15u)
         return fail(KLEOS_EINVAL, "kleos_moe_forward_static_scratch: iP and oP must be 16-byte aligned");
-    kleos_config_t cfg = *user_cfg;
-    if (int rc = kleos_config_derive(&cfg)) return rc;
-    if (const char* why = unsupported_reason(cfg.E, cfg.k)) return fail(KLEOS_EUNSUPPORTED, "%s", why);
-    const DeviceSetup* dev = nullptr;
-    if (int rc = device_setup(&dev)) return rc;
-    if (!dev->gfx950) return fail(KLEOS_EUNSUPPORTED, "the current device is not gfx950: this library is built for MI355X only");
-    LayerParams p{};
-    params_from_config(p, cfg);
-    p.gate_splits = gate_splits_for(cfg.S, cfg.H, cfg.E, cfg.PX, int(cfg.torch_dtype), dev->num_cus);
-    const ArenaLayout L = layout_arena(cfg, p.n_gate_tiles, p.n_super, p.gate_splits);
-    if (L.total > kStaticScratchBytes)
-        return fail(KLEOS_EUNSUPPORTED, "kleos_moe_forward_static_scratch: this configuration needs %zu bytes of library "
-                    "memory, the static scratch holds %zu; use kleos_initialize + kleos_moe_forward", L.total,
-                    kStaticScratchBytes);
-    params_from_arena(p, dev->scratch_ptr, L);
-    bind_buffers(p, cfg, iP, oP);
-    FusedPlan plan;
-    KLEOS_HIP(plan_fused(p, int(cfg.torch_dtype), dev->num_cus, &plan));
-    if (plan.nwg > kMaxWorkgroups) return fail(KLEOS_EUNSUPPORTED, "persistent grid of %u workgroups exceeds %u", plan.nwg, kMaxWorkgroups);
+    StaticCall c;
+    if (int rc = prepare_static_call(user_cfg, c)) return rc;
+    LayerParams& p = c.p;
+    bind_buffers(p, c.cfg, iP, oP);
     // The array keeps what the last call left, of whatever configuration: every counter goes back
     // to zero (a fill kernel, which a stream capture records faithfully), and the launch runs as the
     // first one of a fresh arena.
     hipStream_t s = static_cast<hipStream_t>(stream);
-    const size_t words = (L.zero_end - L.zero_begin) / 4;
-    hipLaunchKernelGGL(zero_words_kernel, dim3(64), dim3(256), 0, s, reinterpret_cast<uint32_t*>(dev->scratch_ptr + L.zero_begin), words);
+    const size_t words = (c.L.zero_end - c.L.zero_begin) / 4;
+    uint32_t* sticky = reinterpret_cast<uint32_t*>(c.dev->scratch_ptr + kStaticScratchUsable);
+    // (every layout starts with the scheduler words, so whatever call came before left its error word here)
+    hipLaunchKernelGGL(zero_words_kernel, dim3(64), dim3(256), 0, s, reinterpret_cast<uint32_t*>(c.dev->scratch_ptr + c.L.zero_begin),
+                       words, (c.L.sched - c.L.zero_begin) / 4 + size_t(sched_error_word()), sticky);
     KLEOS_HIP(hipGetLastError());
     p.epoch = 0;
-    KLEOS_HIP(launch_fused(p, plan, 0, KLEOS_SCHEDULE_AUTO, s));
+    if (g_static_wait_ticks) p.wait_ticks = g_static_wait_ticks;
+    KLEOS_HIP(launch_fused(p, c.plan, g_static_skip, KLEOS_SCHEDULE_AUTO, s));
+    return KLEOS_OK;
+}
+
+extern "C" int kleos_static_scratch_status(void* stream) {
+    DeviceSetup* dev = nullptr;
+    if (int rc = device_setup(&dev)) return rc;
+    KLEOS_HIP(hipStreamSynchronize(static_cast<hipStream_t>(stream)));
+    // the word of the last launch (every layout keeps it at the same place), and the record of the launches before it
+    const size_t error_offset = size_t(sched_error_word()) * 4;
+    uint32_t now = 0, before = 0;
+    KLEOS_HIP(hipMemcpy(&now, dev->scratch_ptr + error_offset, 4, hipMemcpyDeviceToHost));
+    KLEOS_HIP(hipMemcpy(&before, dev->scratch_ptr + kStaticScratchUsable, 4, hipMemcpyDeviceToHost));
+    if (!now && !before) return KLEOS_OK;
+    const uint32_t zero = 0;
+    KLEOS_HIP(hipMemcpy(dev->scratch_ptr + error_offset, &zero, 4, hipMemcpyHostToDevice));
+    KLEOS_HIP(hipMemcpy(dev->scratch_ptr + kStaticScratchUsable, &zero, 4, hipMemcpyHostToDevice));
+    return fail(KLEOS_EHIP, "kleos_moe_forward_static_scratch: a bounded wait of the persistent kernel expired in %s; "
+                            "the outputs of that call are invalid (is the device busy with other kernels, or did calls overlap?)",
+                now ? "the most recent call" : "an earlier call");
+}
+
+extern "C" int kleos_debug_static_scratch_expiry(unsigned long long ticks, uint32_t skip_launch_numbers) {
+    g_static_wait_ticks = ticks;
+    g_static_skip = skip_launch_numbers;
+    return KLEOS_OK;
+}
+
+extern "C" int kleos_debug_map_hip_error(int hip_error) {
+    KLEOS_HIP(static_cast<hipError_t>(hip_error));
     return KLEOS_OK;
 }
 
@@ -299,7 +391,7 @@ extern "C" int kleos_initialize_cfg(const kleos_config_t* user_cfg) {
     KLEOS_HIP_BAIL(hipGetDevice(&c->device));
     {
         // the address of this device's static scratch, for kleos_moe_forward_static_scratch
-        const DeviceSetup* dev = nullptr;
+        DeviceSetup* dev = nullptr;
         if (int rc = device_setup(&dev)) return bail(rc);
     }
     hipDeviceProp_t prop;

@@ -184,7 +184,8 @@ extern "C" int kleos_config_derive(kleos_config_t* c) {
     if (c->hidden_act > KLEOS_ACT_GELU) return fail(KLEOS_EINVAL, "hidden_act must be 0 (relu) or 1 (gelu), got %u", c->hidden_act);
     if (c->torch_dtype > KLEOS_DTYPE_FP16) return fail(KLEOS_EINVAL, "torch_dtype must be 0..3, got %u", c->torch_dtype);
     if (c->torch_dtype == KLEOS_DTYPE_TF32)
-        return fail(KLEOS_EUNSUPPORTED, "torch_dtype 1 (tf32) is unsupported: CDNA4 has no tf32 matrix path; use 0 (fp32), 2 (bf16) or 3 (fp16)");
+        return fail(KLEOS_EUNSUPPORTED, "torch_dtype 1 (tf32, the value the reference ships in kleos_config.json) is unsupported: CDNA4 has no "
+                    "tf32 matrix path; set \"torch_dtype\" to 2 (bf16), 3 (fp16) or 0 (fp32) in the configuration");
     if (c->num_experts < 1) return fail(KLEOS_EINVAL, "num_experts must be >= 1");
     if (c->num_experts > 65535) return fail(KLEOS_EINVAL, "num_experts must be <= 65535 (types.cuh:479), got %u", c->num_experts);
     if (c->expert_top_k < 1) return fail(KLEOS_EINVAL, "expert_top_k must be >= 1");

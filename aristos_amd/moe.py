@@ -39,6 +39,24 @@ def forward_static_scratch(config, iP, oP, stream: int = 0) -> None:
     _capi.check(_capi.lib().kleos_moe_forward_static_scratch(C.byref(st), _ptr(iP), _ptr(oP), stream or None))
 
 
+def static_scratch_prepare(config) -> None:
+    """kleos_static_scratch_prepare: the per-device set-up and the launch plan of `config`, so that a
+    first forward_static_scratch of that layer may be recorded under stream capture."""
+    st = config.to_struct()
+    _capi.check(_capi.lib().kleos_static_scratch_prepare(C.byref(st)))
+
+
+def static_scratch_status(stream: int = 0) -> None:
+    """kleos_static_scratch_status: drains `stream`, raises KleosError (KLEOS_EHIP) if a wait inside a
+    static-scratch forward expired since the last status call."""
+    _capi.check(_capi.lib().kleos_static_scratch_status(stream or None))
+
+
+def debug_static_scratch_expiry(ticks: int, skip_launch_numbers: int) -> None:
+    """Test hook: tick limit and launch-number offset of later static-scratch forwards ((0, 0): normal)."""
+    _capi.check(_capi.lib().kleos_debug_static_scratch_expiry(int(ticks), int(skip_launch_numbers)))
+
+
 def stream_synchronize() -> None:
     _capi.check(_capi.lib().kleos_stream_synchronize())
 

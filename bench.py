@@ -58,6 +58,25 @@ def measured_traffic(workload: str):
     return float(m.group(1)) * 1e9, bool(fp and fp.group(1) == source_fingerprint())
 
 
+PHASED_SKIP, FUSED_SKIP, REHEARSALS = 8, 32, 3
+
+
+def prewarm_protocol(steps: int, warmup: int, pass_ms):
+    """What runs before the timed region, spelled out for the JSON line: the launches of the
+    per-phase measurements (phased and persistent), the rehearsal passes of the whole
+    `warmup` + `steps` pattern, and the per-step latency every pass measured. The first pass is what
+    a caller sees who runs `warmup` + `steps` from cold; the last one is `value`."""
+    phased = PHASED_SKIP + max(64, steps)
+    fused = FUSED_SKIP + max(1536, steps)
+    return {
+        "prewarm_launches": phased + fused + REHEARSALS * (warmup + steps),
+        "prewarm_detail": {"phased_forwards": phased, "persistent_forwards": fused,
+                           "rehearsal_passes": REHEARSALS, "forwards_per_pass": warmup + steps},
+        "pass_ms_per_step": [round(v, 5) for v in pass_ms],
+        "cold_ms_per_step": round(pass_ms[0], 5) if pass_ms else None,
+    }
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -113,19 +132,22 @@ def main() -> int:
         ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         # ---- phased mode first: the same device code, one launch per phase, for per-phase figures
         ka.moe.set_mode(ka.MODE_PHASED)
-        ph_total = ka.moe.forward_host_bench(iP, oP, skip=8, trials=max(64, args.steps))
+        ph_total = ka.moe.forward_host_bench(iP, oP, skip=PHASED_SKIP, trials=max(64, args.steps))
         ph = ka.moe.phase_times()
         # ---- fused mode: the product path. Event-timed on the library stream (the reference's protocol,
         # moe.cuh:160-181: skip launches, then trials launches between two events) ...
         ka.moe.set_mode(ka.MODE_FUSED)
-        ka.moe.forward_host_bench(iP, oP, skip=32, trials=max(1536, args.steps))
+        ka.moe.forward_host_bench(iP, oP, skip=FUSED_SKIP, trials=max(1536, args.steps))
         # ... then, with nothing in between (the device drops its clocks within milliseconds of idling),
         # the timed region: `warmup` forwards, then exactly `steps` forwards, timed by the wall clock (the
         # reported value) and, the same launches, by HIP events on the stream the kernel runs on
         # The protocol runs four times back to back and only the last pass counts: whatever ran before
-        # (nothing, 256 or 1536 launches), the first passes of this launch pattern measure high - at 20
-        # steps about 380, 342 and 337 us per step before the figure settles at 330-334.
-        for rehearsal in (True, True, True, False):
+        # (nothing, 256 or 1536 launches), the first passes of this launch pattern measure high (at 20
+        # steps the first pass reads some 8 % above the fourth). Every pass is reported in the JSON line
+        # (`pass_ms_per_step`; the first as `cold_ms_per_step`), with the count of launches before the
+        # timed region (`prewarm_launches`).
+        pass_ms = []
+        for _ in range(REHEARSALS + 1):
             for _ in range(args.warmup):
                 ka.moe.forward_host(iP, oP)
             ka.moe.stream_synchronize()
@@ -139,6 +161,7 @@ def main() -> int:
             torch.cuda.synchronize()
             wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
             ev_ms = ev0.elapsed_time(ev1) / args.steps
+            pass_ms.append(wall_ms)
         # per-phase figures of the persistent kernel: from the stamps of the last launch and an event-timed run
         ka.moe.forward_host_bench(iP, oP, skip=0, trials=8)
         fused_ph = ka.moe.phase_times()
@@ -201,6 +224,7 @@ def main() -> int:
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": round(wall_ms, 5),
+        **prewarm_protocol(args.steps, args.warmup, pass_ms),
         "higher_is_better": False,
         "scaling": "weak",
         "vs_baseline": None,

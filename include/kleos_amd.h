@@ -139,7 +139,8 @@ int kleos_moe_forward_bench(const void* iP, void* oP, uint32_t skip, uint32_t tr
  * code under HIP stream capture, tight serving loops, harnesses that forbid hipMalloc. The same
  * forward as kleos_moe_forward (persistent launch, KLEOS_SCHEDULE_AUTO), but every library-owned array
  * (routing tables, the activations between the projections, scheduler counters) lives in a fixed
- * array of KLEOS_STATIC_SCRATCH_BYTES bytes in device memory that each GPU holds from the moment the
+ * array of KLEOS_STATIC_SCRATCH_BYTES bytes (the last 256 hold a record of expired waits) in device
+ * memory that each GPU holds from the moment the
  * library is loaded until the process ends. Needs no kleos_initialize and leaves an initialised
  * context alone; calls no hipMalloc / hipFree or any other allocating routine.
  *   cfg:    the JSON keys of the layer (derived fields are recomputed); a configuration whose arrays
@@ -150,10 +151,28 @@ int kleos_moe_forward_bench(const void* iP, void* oP, uint32_t skip, uint32_t tr
  *           stream has drained.
  * All calls on one GPU share that GPU's array: calls that overlap on a GPU (two streams, two
  * threads) race and give wrong results; calls on one stream are ordered and safe, whatever their
- * configurations. An expired in-kernel wait (see kleos_debug_set_wait_ticks) is not reported here.
+ * configurations. The same holds for a kleos_moe_forward in flight on the library stream (which
+ * does not wait for other streams): two persistent grids cannot be resident together, so the call
+ * must not overlap it either. The first call for a layer on a device makes the runtime queries of a
+ * launch plan (function attributes, occupancy) and, on a device's very first call, looks the array's
+ * address up: make it outside stream capture, or call kleos_static_scratch_prepare first. Later calls
+ * for that layer make no runtime queries. An expired in-kernel wait (the device was busy with other
+ * kernels, or calls overlapped) is not reported by this call, which does not synchronise: ask
+ * kleos_static_scratch_status.
  */
 #define KLEOS_STATIC_SCRATCH_BYTES (32u << 20)
 int kleos_moe_forward_static_scratch(const kleos_config_t* cfg, const void* iP, void* oP, void* stream);
+/* No counterpart in the reference. Everything kleos_moe_forward_static_scratch needs before its first
+ * launch of the layer `cfg` on the current device: the address of the device's scratch array and the
+ * launch plan of the layer (kept for the sixteen most recent layers per device). Enqueues nothing,
+ * allocates nothing. For callers whose first forward is recorded under stream capture. */
+int kleos_static_scratch_prepare(const kleos_config_t* cfg);
+/* No counterpart in the reference. Drains `stream` (a hipStream_t; NULL: the default stream), then
+ * reports whether a bounded wait of the persistent kernel expired in any static-scratch call on the
+ * current device since the last status call: KLEOS_OK, or KLEOS_EHIP (the text says whether it was
+ * the most recent call or an earlier one), after which the record is cleared. The outputs of a call
+ * with an expired wait are invalid. Allocates nothing. */
+int kleos_static_scratch_status(void* stream);
 /* Blocks until everything queued on the library stream has finished
  * (cudaStreamSynchronize(kleosStream) in the reference's callers, csrc/main.cu:64-70). */
 int kleos_stream_synchronize(void);
@@ -184,12 +203,18 @@ int kleos_set_schedule(int schedule);
 int kleos_get_schedule(void);
 /* The persistent kernel holds grid-wide barriers, so all its workgroups (one per compute unit) must
  * be resident together. The library sizes the grid from the occupancy the runtime reports for an
- * otherwise idle device; on a device that is busy with other kernels the barriers run into their
- * time limit (see kleos_debug_set_wait_ticks) and the launch is reported as failed. With
- * kleos_set_cooperative_launch(1) the kernel goes through hipLaunchCooperativeKernel instead, which
- * makes the runtime itself check at every launch that the grid fits and return an error if it does not
- * (measured: about 14 us more per launch, which is why it is off by default). The reference launches
- * its persistent kernel plainly (moe.cuh:170, 198) and does not check. */
+ * otherwise idle device. What happens on a device that is busy with other kernels:
+ *   plain launch (default): kleos_moe_forward returns KLEOS_OK; inside the kernel every barrier gives
+ *     up after its time limit (3 s each unless kleos_debug_set_wait_ticks says otherwise), the grid
+ *     drains, and the NEXT synchronising call - kleos_stream_synchronize, kleos_moe_forward_bench,
+ *     kleos_gate_loss - returns KLEOS_EHIP with "a bounded wait on the tile scheduler expired"; the
+ *     outputs of that forward are invalid and the scheduler state has been reset.
+ *   kleos_set_cooperative_launch(1): the kernel goes through hipLaunchCooperativeKernel, the runtime
+ *     itself checks at every launch that the grid fits, and kleos_moe_forward ITSELF returns KLEOS_EHIP
+ *     (the text names hipErrorCooperativeLaunchTooLarge) without launching anything. Measured: about
+ *     14 us more per launch, which is why it is off by default.
+ *   kleos_moe_forward_static_scratch: plain launch; kleos_static_scratch_status reports the expiry.
+ * The reference launches its persistent kernel plainly (moe.cuh:170, 198) and does not check. */
 int kleos_set_cooperative_launch(int on);
 /* The schedule the most recent persistent launch took: KLEOS_SCHEDULE_DYNAMIC or
  * KLEOS_SCHEDULE_STATIC. Synchronises the library stream. KLEOS_ESTATE before the first launch. */
@@ -269,6 +294,17 @@ int kleos_debug_set_wait_ticks(unsigned long long ticks);
  * the next launch expects, every barrier of that launch runs into its time limit, and the launch
  * reports the expiry. For tests of the recovery path (with a small tick limit set first). */
 int kleos_debug_skip_launch_number(void);
+
+/* The tests' handle on kleos_static_scratch_status: later static-scratch calls run with this tick limit
+ * on their in-kernel waits (0: the default) and as launch number `skip_launch_numbers` of their fresh
+ * counters instead of 0, so that with a non-zero skip every barrier runs into the limit, every kernel
+ * still exits, and the status call reports the expiry. (0, 0) restores normal operation. */
+int kleos_debug_static_scratch_expiry(unsigned long long ticks, uint32_t skip_launch_numbers);
+/* The code and message a failed HIP runtime call turns into at this boundary: KLEOS_OK for
+ * hipSuccess (0), else KLEOS_EHIP with the runtime's name and description of `hip_error` in
+ * kleos_last_error(). Touches no device: lets a test pin, for instance, what a refused cooperative
+ * launch (hipErrorCooperativeLaunchTooLarge) looks like to a caller. */
+int kleos_debug_map_hip_error(int hip_error);
 
 /* ---- errors --------------------------------------------------------------------------------- */
 /* Replaces the KLEOS_CHECK_CUDA / KLEOS_ASSERT message conventions (csrc/include/kleos/debug.cuh:

@@ -38,3 +38,14 @@ def test_more_than_one_gpu_is_refused_with_a_message():
     r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
     assert r.returncode != 0
     assert "one GPU" in (r.stdout + r.stderr) or "1 GPU" in (r.stdout + r.stderr) or "single" in (r.stdout + r.stderr).lower()
+
+
+def test_the_json_line_says_what_ran_before_the_timed_region():
+    """`warmup` alone under-reports the warm-up: the line also carries the launches of the per-phase
+    measurements and the rehearsal passes, and what the first (cold) pass measured."""
+    rec = bench.prewarm_protocol(steps=20, warmup=5, pass_ms=[0.3257, 0.3145, 0.2937, 0.3011])
+    assert rec["prewarm_launches"] == (8 + 64) + (32 + 1536) + 3 * (5 + 20)
+    assert rec["cold_ms_per_step"] == 0.3257 and rec["pass_ms_per_step"][-1] == 0.3011
+    assert rec["prewarm_detail"]["rehearsal_passes"] == 3 and len(rec["pass_ms_per_step"]) == 4
+    src = open(os.path.join(ROOT, "bench.py")).read()
+    assert "**prewarm_protocol(args.steps, args.warmup, pass_ms)" in src   # the keys reach the printed line

@@ -60,3 +60,15 @@ def test_bench_refuses_more_than_one_gpu():
     proc = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
     assert proc.returncode == 2
     assert "single-GPU" in proc.stderr and proc.stdout.strip() == ""
+
+
+def test_a_refused_cooperative_launch_maps_to_kleos_ehip():
+    """With kleos_set_cooperative_launch(1) a grid that cannot be resident is refused by the runtime at
+    launch (hipErrorCooperativeLaunchTooLarge, 720) and kleos_moe_forward itself returns KLEOS_EHIP with
+    the runtime's name of the error; hipSuccess maps to KLEOS_OK. The mapping touches no device."""
+    lib = _capi.lib()
+    assert lib.kleos_debug_map_hip_error(0) == _capi.KLEOS_OK
+    assert lib.kleos_debug_map_hip_error(720) == _capi.KLEOS_EHIP
+    assert "hipErrorCooperativeLaunchTooLarge" in lib.kleos_last_error().decode()
+    assert lib.kleos_debug_map_hip_error(2) == _capi.KLEOS_EHIP
+    assert "hipErrorOutOfMemory" in lib.kleos_last_error().decode()

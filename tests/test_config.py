@@ -25,6 +25,10 @@ def test_parse_shipped_config_keys():
     with pytest.raises(ka.KleosError) as ei:
         cfg.derive()
     assert ei.value.code == _capi.KLEOS_EUNSUPPORTED and "tf32" in ei.value.message
+    # the message names the remedy, and the remedy works: the same keys with torch_dtype 2 are the headline layer
+    assert 'set "torch_dtype" to 2' in ei.value.message
+    d = ka.KleosConfig.from_json_text(json.dumps({**SHIPPED, "torch_dtype": 2})).derive()
+    assert (d.S, d.H, d.I, d.E, d.k, d.EC) == (8192, 2048, 2048, 64, 2, 256)
 
 
 @pytest.mark.parametrize("name,S,PX,EC,pEC,in_elems", [

@@ -26,6 +26,25 @@ TOL_LOGIT = {0: 2e-5, 2: 2e-5, 3: 2e-5}    # absolute, fp32 accumulation of exac
 TOL_PROB = {0: 2e-6, 2: 4e-3, 3: 5e-4}     # gateOut: fp32 exp/div ulps, or one bf16 / fp16 rounding
 
 
+def tol_out(c):
+    """moeOut. The reference adds the k scaled expert rows of a token into the output one by one in
+    Element (atomicAdd, processor.cuh:157,165), and so does the oracle: k roundings of the running sum,
+    a random walk of about u * sqrt(k / 3) relative (u = 2^-9 for bf16: 0.96 % at k = 72), while the GPU
+    sums in fp32 and rounds once. Up to k = 16 that stays inside the stated tolerance; above, the bound
+    grows with sqrt(k) like the walk it allows for (k = 72 in bf16 measures 1.2 %)."""
+    return TOL_OUT[c.dtype] * max(1.0, (c.k / 16.0) ** 0.5)
+
+
+def tol_prob(c):
+    """gateOut. In fp32 the softmax denominator is a sum of E terms that the GPU adds in a tree over lanes
+    and the oracle in index order (gate.cuh:574-580): next to a probability close to 1 the two orders
+    differ by about 2^-24 * sqrt(E) (500 experts with one dominant expert measure 2.4e-6). The bound
+    grows with sqrt(E) above 128 experts; the 16-bit Elements are bounded by their own rounding."""
+    if c.dtype == 0:
+        return TOL_PROB[0] * max(1.0, (c.E / 128.0) ** 0.5)
+    return TOL_PROB[c.dtype]
+
+
 def _to_device(c, iP_np):
     if c.dtype in (2, 3):
         return torch.from_numpy(iP_np.view(np.int16)).cuda().view(torch.bfloat16 if c.dtype == 2 else torch.float16)
@@ -87,14 +106,14 @@ def check_against_oracle(c, keys, iP_np, mode, launches=1, token_mask=None, logi
     assert np.isfinite(out).all(), "the layer left output elements unwritten"
     gate_out = out[:c.S * c.PX].reshape(c.S, c.PX)
     moe_out = out[c.S * c.PX:].reshape(c.S, c.H)
-    assert np.abs(gate_out - ref["gate_out"]).max() < TOL_PROB[c.dtype]
+    assert np.abs(gate_out - ref["gate_out"]).max() < tol_prob(c)
     assert (gate_out[:, c.E:] == 0).all()
     if token_mask is not None:
         sel = token_mask.astype(bool)
         err = rel_fro(moe_out[sel], ref["moe_out"][sel])
     else:
         err = rel_fro(moe_out, ref["moe_out"])
-    assert err < TOL_OUT[c.dtype], f"relative Frobenius error {err}"
+    assert err < tol_out(c), f"relative Frobenius error {err}"
     # tokens dropped by every expert are zero rows
     all_dropped = (v["topk_slot"] < 0).all(axis=1)
     assert (moe_out[all_dropped] == 0).all()
@@ -144,6 +163,8 @@ CASES = [
     (256, 128, 64, 130, 8, 1.0, 1, 0, 2, 0.0),     # E > 128 (gate handles up to 256 experts)
     (256, 128, 64, 256, 8, 1.0, 1, 0, 2, 0.0),     # E = 256, top-8
     (128, 128, 64, 96, 72, 1.0, 1, 0, 3, 0.0),     # fp16, 64 < E <= 256 with k > 64: more picks per token than a wavefront has lanes
+    (128, 128, 64, 96, 72, 1.0, 1, 0, 2, 0.0),     # the same in bf16: 72 Element additions per output row in the oracle (tol_out)
+    (256, 448, 320, 500, 20, 1.25, 0, 0, 0, 0.1),  # fp32, 500 experts, top-20, no dropping: the softmax denominator's 500 terms (tol_prob)
     (256, 128, 64, 200, 5, 1.5, 1, 0, 3, 0.1),     # fp16, E = 200 (padded to 256 columns, not a multiple of 16)
     (256, 128, 192, 8, 2, 1.0, 1, 1, 0, 0.1),      # fp32 + gelu
     (256, 64, 64, 24, 3, 1.0, 1, 0, 0, 0.0),       # fp32, E = 24

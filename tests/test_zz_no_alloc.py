@@ -135,3 +135,62 @@ def test_static_scratch_forward_replays_from_a_graph():
         # eager work on the same array, of another shape, between the replays
         ka.moe.forward_static_scratch(other, iP2, oP2)
         torch.cuda.synchronize()
+
+
+def test_static_scratch_status_reports_an_expired_wait():
+    """An expired in-kernel wait of a static-scratch forward is on record until the status call has
+    reported it. The expiry is provoked from the host (a 0.2 ms limit on every wait, and counters that
+    lag the launch number by one launch, so that no barrier is ever complete); every kernel exits
+    normally, and the next forward gives the right bits again."""
+    keys = _keys(1024, 256, 512, 16, 2)
+    c, iP = _device_inputs(keys, 71)
+    d, ref = _existing_entry_point(keys, iP)
+    ref = _bits(c, ref)
+    oP = synth.alloc_outputs(d)
+    ka.moe.forward_static_scratch(keys, iP, oP)
+    ka.moe.static_scratch_status()            # nothing expired
+    try:
+        ka.moe.debug_static_scratch_expiry(20000, 1)
+        ka.moe.forward_static_scratch(keys, iP, oP)
+        with pytest.raises(ka.KleosError) as ei:
+            ka.moe.static_scratch_status()
+        assert ei.value.code == _capi.KLEOS_EHIP and "the most recent call" in ei.value.message, ei.value.message
+        ka.moe.static_scratch_status()        # the record was cleared
+        # a failed call followed by a good one: the fill kernel of the good call keeps the record
+        ka.moe.forward_static_scratch(keys, iP, oP)
+        ka.moe.debug_static_scratch_expiry(0, 0)
+        oP.fill_(float("nan"))
+        ka.moe.forward_static_scratch(keys, iP, oP)
+        with pytest.raises(ka.KleosError) as ei:
+            ka.moe.static_scratch_status()
+        assert ei.value.code == _capi.KLEOS_EHIP and "an earlier call" in ei.value.message, ei.value.message
+        np.testing.assert_array_equal(_bits(c, oP), ref)   # the good call itself was fine
+    finally:
+        ka.moe.debug_static_scratch_expiry(0, 0)
+    ka.moe.static_scratch_status()
+    oP.fill_(float("nan"))
+    ka.moe.forward_static_scratch(keys, iP, oP)
+    ka.moe.static_scratch_status()
+    np.testing.assert_array_equal(_bits(c, oP), ref)
+
+
+def test_static_scratch_first_call_of_a_layer_under_capture():
+    """After kleos_static_scratch_prepare the first forward of a layer may be recorded under stream
+    capture: the launch plan is looked up, nothing queries the runtime."""
+    keys = _keys(512, 192, 320, 12, 3)       # a layer no other test of this file runs
+    c, iP = _device_inputs(keys, 74)
+    d, ref = _existing_entry_point(keys, iP)
+    ref = _bits(c, ref)
+    oP = synth.alloc_outputs(d)
+    ka.moe.static_scratch_prepare(keys)
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        ka.moe.forward_static_scratch(keys, iP, oP, stream=torch.cuda.current_stream().cuda_stream)
+    for _ in range(3):
+        oP.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        np.testing.assert_array_equal(_bits(c, oP), ref)
+    ka.moe.static_scratch_status()
