@@ -20,7 +20,7 @@ HIPCC_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wextra", "-Wno-unused-parameter", "-Wno-pass-failed",
 ]
-SOURCES = ["config.cpp", "capi.hip", "kernels.hip"]
+SOURCES = ["config.cpp", "capi.hip", "kernels.hip", "kernels_f32.hip", "kernels_bf16.hip", "kernels_f16.hip"]
 
 
 def _hipcc() -> str:
@@ -40,10 +40,18 @@ def _run(cmd: list[str]) -> None:
         sys.stderr.write(err + "\n")
 
 
-def build_library(driver: bool = True) -> str:
-    """Compiles every HIP source into libkleos_amd.so (and the C++ driver); returns the library path."""
+def build_library(driver: bool = True, jobs: int = 6) -> str:
+    """Compiles every HIP source into libkleos_amd.so (and the C++ driver); returns the library path.
+    The sources are compiled side by side (one hipcc process each, objects under aristos_amd/build/),
+    then linked."""
+    from concurrent.futures import ThreadPoolExecutor
+    obj_dir = os.path.join(PKG_DIR, "build")
+    os.makedirs(obj_dir, exist_ok=True)
+    objs = [os.path.join(obj_dir, os.path.splitext(src)[0] + ".o") for src in SOURCES]
+    with ThreadPoolExecutor(max_workers=max(1, min(jobs, len(SOURCES)))) as pool:
+        list(pool.map(lambda so: _run([_hipcc(), *HIPCC_FLAGS, "-c", so[0], "-o", so[1]]), zip(SOURCES, objs)))
     tmp = LIB_PATH + ".tmp"
-    _run([_hipcc(), *HIPCC_FLAGS, "-shared", *SOURCES, "-o", tmp])
+    _run([_hipcc(), "--offload-arch=gfx950", "-shared", *objs, "-o", tmp])
     os.replace(tmp, LIB_PATH)
     if driver:
         _run([_hipcc(), *HIPCC_FLAGS, "main.cpp", "-o", DRIVER_PATH, f"-L{PKG_DIR}", "-lkleos_amd",

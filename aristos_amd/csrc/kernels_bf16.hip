@@ -1,0 +1,6 @@
+// The kernels of the MoE layer forward for Element = bf16_t (see kernels_impl.hpp).
+#include "kernels_impl.hpp"
+
+namespace kleos_amd {
+KLEOS_INSTANTIATE_ELEMENT(bf16_t)
+}  // namespace kleos_amd

@@ -96,14 +96,15 @@ def test_static_scratch_forward_matches_the_allocating_one():
 
 
 def test_static_scratch_refuses_what_does_not_fit():
-    """The headline layer needs about 134 MB of library arrays: beyond the 32 MiB the scratch holds."""
+    """The headline layer needs about 137 MB of library arrays: beyond what the 32 MiB scratch holds
+    (all of it but the 256 bytes at its end that keep the record of expired waits)."""
     keys = synth.WORKLOADS["headline_e64_zipf"].config
     dummy = torch.zeros(64, dtype=torch.bfloat16, device="cuda")
     st = keys.to_struct()
     rc = _capi.lib().kleos_moe_forward_static_scratch(ctypes.byref(st), dummy.data_ptr(), dummy.data_ptr(), None)
     assert rc == _capi.KLEOS_EUNSUPPORTED
     msg = _capi.lib().kleos_last_error().decode()
-    assert "static scratch holds 33554432" in msg, msg
+    assert f"static scratch holds {(32 << 20) - 256}" in msg, msg
     torch.cuda.synchronize()
 
 
