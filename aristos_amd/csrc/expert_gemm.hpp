@@ -152,6 +152,15 @@ __device__ __forceinline__ void epilogue16(const TileOut& t, f32x16 (&acc)[WN / 
     else epilogue16_act<E, WM, WN, WAVES_N, 2>(t, acc, stage_mem, bias_mem);
 }
 
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>), in this order.
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (N > 0) {
+        static_for<N - 1>(f);
+        f(std::integral_constant<int, N - 1>{});
+    }
+}
+
 // STREAM_B: the weight rows are loaded with the non-temporal cache policy: read once (or by a
 // neighbour at the same moment), they pass through the L2 without displacing the activation rows
 // that are shared (7.0 against 6.4 TB/s on a read-only stream of this shape).
@@ -160,7 +169,14 @@ __device__ __forceinline__ void epilogue16(const TileOut& t, f32x16 (&acc)[WN / 
 // its matrix work (headline shape: 301 against 315 us for the expert phase); where the matrix work
 // dominates the extra barrier costs more than the earlier loads bring (8-expert shape with hidden
 // size 4096: 4.22 against 4.03 ms).
-template <typename E, int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES, bool STREAM_B, bool AHEAD2>
+// SPREAD (with AHEAD2): when the loads of a slice are issued. 0: all of them behind the matrix
+// instructions of the last K step of the slice two before it, which frees their stage. Otherwise
+// only the first of them go there and the rest behind the first three K steps of the next slice
+// (spread_count): the CU's load path takes in one 1 KB load about every 36 clocks while all CUs
+// stream, so the 64 loads of a slice issued by eight wavefronts inside one K step hold every
+// wavefront - and with it its matrix instructions, which sit behind the loads in program order -
+// for as long as four K steps of matrix work take.
+template <typename E, int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES, bool STREAM_B, bool AHEAD2, int SPREAD = 0>
 struct Gemm16 {
     typedef typename Elem16<E>::vec8 vec8;
     typedef typename Elem16<E>::vec4 vec4;
@@ -182,6 +198,23 @@ struct Gemm16 {
     static constexpr int kSliceK = BK;                             // values of K per slice
     static constexpr int kSteps = BK / 16;                         // matrix instructions consume 16 values of K
     static constexpr int kPanelRows = kEpiloguePanelRows;          // epilogue staging: 32 rows x 64 columns per wavefront
+    // loads of a slice (per wavefront) issued at the last K step of the slice two before it [0] and at
+    // K steps 0, 1, 2 of the slice before it [1..3]; SPREAD >= 10: weight rows before activation rows
+    static constexpr int kPolicy = SPREAD % 10;
+    static constexpr bool kWeightsFirst = SPREAD >= 10;
+    static constexpr int spread_count(int i) {
+        constexpr int L = LA + LB;
+        switch (kPolicy) {
+            case 1: return i < 2 ? L / 2 : 0;                                   // 4 4 0 0
+            case 2: return i == 0 || i == 1 ? (3 * L) / 8 : (i == 2 ? L - 2 * ((3 * L) / 8) : 0);   // 3 3 2 0
+            case 3: return L / 4;                                               // 2 2 2 2
+            case 4: return i == 0 ? L / 2 : (i < 3 ? L / 4 : 0);                // 4 2 2 0
+            case 5: return i == 0 ? L / 4 : (i < 3 ? (3 * L) / 8 : 0);          // 2 3 3 0
+            default: return i == 0 ? L : 0;                                     // all at once
+        }
+    }
+    static_assert(SPREAD == 0 || (AHEAD2 && (LA + LB) % 8 == 0));
+    static_assert(spread_count(0) + spread_count(1) + spread_count(2) + spread_count(3) == LA + LB);
     static_assert(BK == 32 || BK == 64);
     static_assert(!AHEAD2 || STAGES == 2);
     static_assert(STAGES >= 2 && STAGES <= 4);
@@ -226,6 +259,29 @@ struct Gemm16 {
         for (int i = 0; i < LB; ++i)
             __builtin_amdgcn_global_load_lds((global_cptr)(t.pb[i] + k0), (lds_ptr)(sb + 1024 * (wave + kWaves * i)), 16, 0,
                                              STREAM_B ? kNonTemporal : 0);
+    }
+
+    // Load number j (0 <= j < LA + LB) of K slice kt in the order the policy issues them.
+    static __device__ __forceinline__ void issue_one(const Tile& t, char* sa, char* sb, uint32_t k0, int j) {
+        const int wave = threadIdx.x >> 6;
+        const bool is_w = kWeightsFirst ? j < LB : j >= LA;
+        const int i = kWeightsFirst ? (j < LB ? j : j - LB) : (j < LA ? j : j - LA);
+        if (is_w)
+            __builtin_amdgcn_global_load_lds((global_cptr)(t.pb[i] + k0), (lds_ptr)(sb + 1024 * (wave + kWaves * i)), 16, 0,
+                                             STREAM_B ? kNonTemporal : 0);
+        else
+            __builtin_amdgcn_global_load_lds((global_cptr)(t.pa[i] + k0), (lds_ptr)(sa + 1024 * (wave + kWaves * i)), 16, 0, 0);
+    }
+    // Loads first .. first + count - 1 of K slice kt.
+    template <int FIRST, int COUNT>
+    static __device__ __forceinline__ void issue_range(const Tile& t, char* smem, uint32_t kt) {
+        char* sa = smem + stage_of(t, kt) * kStage;
+        char* sb = sa + kABytes;
+        uint32_t slice = kt + t.k_first;
+        slice = slice >= t.k_tiles ? slice - t.k_tiles : slice;
+        const uint32_t k0 = slice * BK;
+#pragma unroll
+        for (int j = 0; j < COUNT; ++j) issue_one(t, sa, sb, k0, FIRST + j);
     }
 
     // Per-lane source addresses, the load of the bias into LDS slot `bias_slot`, then the loads of
@@ -295,16 +351,18 @@ struct Gemm16 {
             // every slice into LDS at the same points of the same sequence of barriers as the others,
             // and leaves the fragment reads and the matrix instructions out.
             if constexpr (AHEAD2) {
+                constexpr int N0 = spread_count(0);
                 asm volatile("s_barrier" ::: "memory");
-                if (t.k_tiles > 1) issue_slice(t, smem, 1);
+                if (t.k_tiles > 1) issue_range<0, N0>(t, smem, 1);
                 for (uint32_t kt = 0; kt < t.k_tiles; ++kt) {
-                    if (kt + 1 < t.k_tiles) wait_vmcnt<kLoadsPerSlice>();
+                    if (kt + 1 < t.k_tiles) wait_vmcnt<N0>();
                     else wait_vmcnt<0>();
                     asm volatile("s_barrier" ::: "memory");
                     if (kt == 0) after_first_barrier();
+                    if (kt + 1 < t.k_tiles) issue_range<N0, LA + LB - N0>(t, smem, kt + 1);
                     if (kt + 2 < t.k_tiles) {
                         asm volatile("s_barrier" ::: "memory");
-                        issue_slice(t, smem, kt + 2);
+                        issue_range<0, N0>(t, smem, kt + 2);
                     }
                 }
             } else {
@@ -360,8 +418,12 @@ struct Gemm16 {
         // 3.47 with the loads interleaved too; with operands resident in L2 3.49, 2.96 and 2.72).
         // LOADS is a compile-time switch: a branch around matrix instructions makes the compiler keep
         // two copies of the accumulators.
-        auto kstep = [&](const char* st, int ks, auto loads_tag, const SliceLoads& l, int load_base) {
-            constexpr bool LOADS = decltype(loads_tag)::value;
+        // `first_tag`, `count_tag`: the K step carries the loads first .. first + count - 1 of the slice `l`
+        // describes, evenly spaced behind its matrix instructions (count 0: none).
+        auto kstep = [&](const char* st, int ks, const SliceLoads& l, auto first_tag, auto count_tag) {
+            constexpr int FIRST = decltype(first_tag)::value, COUNT = decltype(count_tag)::value;
+            static_assert(COUNT <= TN * TM);
+            constexpr int kEvery = (TN * TM) / (COUNT > 0 ? COUNT : 1);
 #pragma unroll
             for (int i = 0; i < TN * TM; ++i) {
                 __builtin_amdgcn_sched_barrier(0);
@@ -372,56 +434,63 @@ struct Gemm16 {
                     if (i < TN) fw[nb][i] = __builtin_bit_cast(vec8, load16(st + (base_w ^ ((ks + 1) << 5)) + i * 32 * kRowBytes));
                     else if (i < TN + TM) fx[nb][i - TN] = __builtin_bit_cast(vec8, load16(st + (base_x ^ ((ks + 1) << 5)) + (i - TN) * 32 * kRowBytes));
                 }
-                if constexpr (LOADS) {
-                    const int li = load_base + i;
-                    if (li < LA)
-                        __builtin_amdgcn_global_load_lds((global_cptr)(t.pa[li] + l.k0), (lds_ptr)(l.sa + 1024 * (wave + kWaves * li)), 16, 0, 0);
-                    else if (li < LA + LB)
-                        __builtin_amdgcn_global_load_lds((global_cptr)(t.pb[li - LA] + l.k0), (lds_ptr)(l.sb + 1024 * (wave + kWaves * (li - LA))), 16,
-                                                         0, STREAM_B ? kNonTemporal : 0);
+                if constexpr (COUNT > 0) {
+                    if (i % kEvery == 0 && i / kEvery < COUNT) {
+                        if constexpr (AHEAD2) {
+                            issue_one(t, l.sa, l.sb, l.k0, FIRST + i / kEvery);
+                        } else {
+                            const int li = FIRST + i / kEvery;
+                            if (li < LA)
+                                __builtin_amdgcn_global_load_lds((global_cptr)(t.pa[li] + l.k0), (lds_ptr)(l.sa + 1024 * (wave + kWaves * li)), 16, 0, 0);
+                            else if (li < LA + LB)
+                                __builtin_amdgcn_global_load_lds((global_cptr)(t.pb[li - LA] + l.k0), (lds_ptr)(l.sb + 1024 * (wave + kWaves * (li - LA))), 16,
+                                                                 0, STREAM_B ? kNonTemporal : 0);
+                        }
+                    }
                 }
             }
             __builtin_amdgcn_sched_barrier(0);
         };
-        constexpr std::true_type with_loads{};
-        constexpr std::false_type without_loads{};
         static_assert(TN + TM <= TN * TM, "a K step has a matrix instruction for every fragment read");
         if constexpr (AHEAD2) {
             static_assert(LA + LB <= TN * TM, "the loads of a slice fit behind the matrix instructions of one K step");
+            static_assert(kSteps == 4);
+            constexpr int N0 = spread_count(0), N1 = spread_count(1), N2 = spread_count(2), N3 = spread_count(3);
             // Slice 0 was requested by begin(). Every wavefront has left the previous tile's epilogue,
-            // which staged its output in the stage slice 1 goes to.
+            // which staged its output in the stage slice 1 goes to: its first loads go out here, the
+            // others behind the first K steps of slice 0.
             asm volatile("s_barrier" ::: "memory");
-            if (t.k_tiles > 1) issue_slice(t, smem, 1);
-            auto top = [&](uint32_t kt) {
-                // this wavefront's loads of slice kt are complete once only those of slice kt+1 are
-                // outstanding (the stores of the previous tile's epilogue are older than both)
-                if (kt + 1 < t.k_tiles) wait_vmcnt<kLoadsPerSlice>();
+            if (t.k_tiles > 1) issue_range<0, N0>(t, smem, 1);
+            // One slice: `next_tag` - slice kt+1 exists (its loads N0 .. are issued behind K steps 0 to 2),
+            // `next2_tag` - slice kt+2 exists (its first N0 loads go behind the last K step, into the
+            // stage of slice kt, once every wavefront has read its last fragments of it).
+            auto slice = [&](uint32_t kt, auto next_tag, auto next2_tag) {
+                constexpr bool NEXT = decltype(next_tag)::value, NEXT2 = decltype(next2_tag)::value;
+                // this wavefront's loads of slice kt are complete once only the first N0 of slice kt+1
+                // are outstanding (the stores of the previous tile's epilogue are older than both)
+                if constexpr (NEXT) wait_vmcnt<N0>();
                 else wait_vmcnt<0>();
                 asm volatile("s_barrier" ::: "memory");   // every wavefront's share of slice kt is in LDS
                 if (kt == 0) after_first_barrier();
+                const char* st = smem + stage_of(t, kt) * kStage;
+                read_fragments(st, 0);
+                const SliceLoads l1 = NEXT ? loads_of(kt + 1) : SliceLoads{};
+                kstep(st, 0, l1, std::integral_constant<int, N0>{}, std::integral_constant<int, NEXT ? N1 : 0>{});
+                kstep(st, 1, l1, std::integral_constant<int, N0 + N1>{}, std::integral_constant<int, NEXT ? N2 : 0>{});
+                kstep(st, 2, l1, std::integral_constant<int, N0 + N1 + N2>{}, std::integral_constant<int, NEXT ? N3 : 0>{});
+                if constexpr (NEXT2) {
+                    // this wavefront's last reads of the stage have returned; once that holds for every
+                    // wavefront the stage takes slice kt+2
+                    __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0)
+                    asm volatile("s_barrier" ::: "memory");
+                }
+                const SliceLoads l2 = NEXT2 ? loads_of(kt + 2) : SliceLoads{};
+                kstep(st, 3, l2, std::integral_constant<int, 0>{}, std::integral_constant<int, NEXT2 ? N0 : 0>{});
             };
             const uint32_t ahead = t.k_tiles >= 2 ? t.k_tiles - 2 : 0u;   // slices that request slice kt+2
-            for (uint32_t kt = 0; kt < ahead; ++kt) {
-                top(kt);
-                const char* st = smem + stage_of(t, kt) * kStage;
-                read_fragments(st, 0);
-                const SliceLoads l = loads_of(kt + 2);
-#pragma unroll
-                for (int ks = 0; ks + 1 < kSteps; ++ks) kstep(st, ks, without_loads, l, 0);
-                // this wavefront's last reads of the stage have returned; once that holds for every
-                // wavefront the stage takes slice kt+2
-                __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0)
-                asm volatile("s_barrier" ::: "memory");
-                kstep(st, kSteps - 1, with_loads, l, 0);
-            }
-            for (uint32_t kt = ahead; kt < t.k_tiles; ++kt) {
-                top(kt);
-                const char* st = smem + stage_of(t, kt) * kStage;
-                read_fragments(st, 0);
-                const SliceLoads l{};
-#pragma unroll
-                for (int ks = 0; ks < kSteps; ++ks) kstep(st, ks, without_loads, l, 0);
-            }
+            for (uint32_t kt = 0; kt < ahead; ++kt) slice(kt, std::true_type{}, std::true_type{});
+            if (t.k_tiles >= 2) slice(t.k_tiles - 2, std::true_type{}, std::false_type{});
+            slice(t.k_tiles - 1, std::false_type{}, std::false_type{});
         } else {
             static_assert(LA + LB <= kSteps * TN * TM, "the loads of a slice fit behind the matrix instructions of a slice");
             auto top = [&](uint32_t kt) {
@@ -436,22 +505,28 @@ struct Gemm16 {
                 asm volatile("s_barrier" ::: "memory");
                 if (kt == 0) after_first_barrier();
             };
+            // K step ks carries the loads ks * TN * TM ... of the slice STAGES-1 ahead, one behind each
+            // matrix instruction, until they run out
+            auto ksteps = [&](const char* st, const SliceLoads& l, auto loads_tag) {
+                static_for<kSteps>([&](auto ks_tag) {
+                    constexpr int ks = decltype(ks_tag)::value;
+                    constexpr int left = LA + LB - ks * TN * TM;
+                    constexpr int count = !decltype(loads_tag)::value || left <= 0 ? 0 : (left < TN * TM ? left : TN * TM);
+                    kstep(st, ks, l, std::integral_constant<int, ks * TN * TM>{}, std::integral_constant<int, count>{});
+                });
+            };
             const uint32_t ahead = t.k_tiles >= uint32_t(STAGES - 1) ? t.k_tiles - (STAGES - 1) : 0u;   // slices that request a later one
             for (uint32_t kt = 0; kt < ahead; ++kt) {
                 top(kt);
                 const char* st = smem + stage_of(t, kt) * kStage;
                 read_fragments(st, 0);
-                const SliceLoads l = loads_of(kt + STAGES - 1);
-#pragma unroll
-                for (int ks = 0; ks < kSteps; ++ks) kstep(st, ks, with_loads, l, ks * TN * TM);
+                ksteps(st, loads_of(kt + STAGES - 1), std::true_type{});
             }
             for (uint32_t kt = ahead; kt < t.k_tiles; ++kt) {
                 top(kt);
                 const char* st = smem + stage_of(t, kt) * kStage;
                 read_fragments(st, 0);
-                const SliceLoads l{};
-#pragma unroll
-                for (int ks = 0; ks < kSteps; ++ks) kstep(st, ks, without_loads, l, 0);
+                ksteps(st, SliceLoads{}, std::false_type{});
             }
         }
     }
@@ -513,8 +588,13 @@ struct Gemm16 {
 };
 
 // ------------------------------------------------------------------------------------------------
-// fp32, vector ALU. 64 x 64 x 16 tile, 256 threads, 4 x 4 outputs per thread, K summed in
-// ascending order. Serves the fp32 configuration, whose sizes are small.
+// fp32, matrix cores. 64 x 64 tile, 256 threads = 2 x 2 wavefronts of 32 x 32, K in slices of 16
+// through LDS (k-major, rows padded to 68 words: the transposing writes and the operand reads both
+// spread over the banks), one 32x32x2 fp32 matrix instruction per two values of K: the weight rows
+// are its row operand and the activation rows its column operand, as in the 16-bit tiles, so a
+// lane owns 4 consecutive output columns of one output row. K is summed in ascending order, two
+// values per instruction - the same order in every launch mode. Serves the fp32 configuration,
+// whose sizes are small.
 // ------------------------------------------------------------------------------------------------
 constexpr int kF32Tile = 64, kF32BK = 16, kF32Pad = 68;
 constexpr int gemm_f32_smem_bytes() { return 2 * kF32BK * kF32Pad * 4; }
@@ -530,7 +610,9 @@ __device__ __forceinline__ void gemm_tile_f32(
     float (*Bs)[kF32Pad] = reinterpret_cast<float (*)[kF32Pad]>(smem + kF32BK * kF32Pad * 4);
     const int tid = threadIdx.x;
     const int ld_row = tid >> 2, ld_kq = tid & 3;
-    const int ty = tid >> 4, tx = tid & 15;
+    const int wave = tid >> 6, lane = tid & 63;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int fr_row = lane & 31, fr_half = lane >> 5;
 
     const float* pa = nullptr;
     const float* pb = nullptr;
@@ -545,7 +627,9 @@ __device__ __forceinline__ void gemm_tile_f32(
     }
     if (uint32_t(ld_row) < n_valid) pb = b_base + size_t(ld_row) * ldb + ld_kq * 4;
 
-    float acc[4][4] = {};
+    f32x16 acc;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[v] = 0.f;
     for (uint32_t k0 = 0; k0 < K; k0 += kF32BK) {
         const f32x4 va = pa ? *reinterpret_cast<const f32x4*>(pa + k0) : f32x4{0.f, 0.f, 0.f, 0.f};
         const f32x4 vb = pb ? *reinterpret_cast<const f32x4*>(pb + k0) : f32x4{0.f, 0.f, 0.f, 0.f};
@@ -557,25 +641,31 @@ __device__ __forceinline__ void gemm_tile_f32(
         }
         __syncthreads();
 #pragma unroll
-        for (int kk = 0; kk < kF32BK; ++kk) {
-            float a[4], b[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) { a[i] = As[kk][ty * 4 + i]; b[i] = Bs[kk][tx * 4 + i]; }
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-#pragma unroll
-                for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+        for (int kk = 0; kk < kF32BK; kk += 2) {
+            // lanes 0-31 bring K value kk, lanes 32-63 K value kk + 1
+            const float w = Bs[kk + fr_half][wn * 32 + fr_row];
+            const float x = As[kk + fr_half][wm * 32 + fr_row];
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(w, x, acc, 0, 0, 0);
         }
     }
+    // acc[v]: output row m = wm * 32 + lane % 32, column n = wn * 32 + 8 (v / 4) + 4 (lane / 32) + v % 4
+    const uint32_t m = wm * 32 + fr_row;
+    if (m < m_valid) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const uint32_t m = ty * 4 + i;
-        if (m >= m_valid) continue;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const uint32_t n = tx * 4 + j;
+        for (int q = 0; q < 4; ++q) {
+            const uint32_t n0 = wn * 32 + 8 * q + 4 * fr_half;
+            float* dst = c_base + size_t(m) * ldc + n0;
             // read by other workgroups later in the same launch: written through the L2
-            if (n < n_valid) store_through(c_base + size_t(m) * ldc + n, activate<ACT>(acc[i][j] + bias[n]));
+            if (n0 + 4 <= n_valid && ((reinterpret_cast<uintptr_t>(dst) & 15u) == 0)) {
+                f32x4 o;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) o[j] = activate<ACT>(acc[4 * q + j] + bias[n0 + j]);
+                store16_through(dst, __builtin_bit_cast(u32x4, o));
+            } else {
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    if (n0 + j < n_valid) store_through(dst + j, activate<ACT>(acc[4 * q + j] + bias[n0 + j]));
+            }
         }
     }
 }

@@ -53,11 +53,33 @@ constexpr int kXcds = 8;
 // Variants 0 and 1 load their weight rows non-temporally (headline 378 against 390 us per forward,
 // the 16-expert shape 192 against 196, the 256-expert shape 3.43 against 3.48 ms); variant 2, whose
 // weight tiles are shared by eight workgroups and more, does not (4.06 against 4.01 ms with it).
+// (The three choices below can be overridden on the compiler's command line for measurements.)
+#ifndef KLEOS_TUNE_V0_SPREAD
+#define KLEOS_TUNE_V0_SPREAD 2       // variant 0: loads of a slice issued 3 + 3 + 2 over three K steps
+#endif
+#ifndef KLEOS_TUNE_V2_SPREAD
+#define KLEOS_TUNE_V2_SPREAD 1       // variant 2: two slices ahead, 4 + 4 over two K steps; -1: one slice ahead
+#endif
+#ifndef KLEOS_TUNE_MIXED_HEIGHTS
+#define KLEOS_TUNE_MIXED_HEIGHTS 1   // variant 2: 128-row tiles for last row blocks of at most 128 rows
+#endif
 template <typename E, int V>
-using GemmCfg = std::conditional_t<V == 0, Gemm16<E, 256, 256, 4, 2, 64, 2, true, true>,
-                std::conditional_t<V == 1, Gemm16<E, 128, 256, 2, 4, 64, 3, true, false>, Gemm16<E, 256, 256, 2, 4, 64, 2, false, false>>>;
+using GemmCfg = std::conditional_t<V == 0, Gemm16<E, 256, 256, 4, 2, 64, 2, true, true, KLEOS_TUNE_V0_SPREAD>,
+                std::conditional_t<V == 1, Gemm16<E, 128, 256, 2, 4, 64, 3, true, false>,
+                                   Gemm16<E, 256, 256, 2, 4, 64, 2, false, (KLEOS_TUNE_V2_SPREAD >= 0), (KLEOS_TUNE_V2_SPREAD >= 0 ? KLEOS_TUNE_V2_SPREAD : 0)>>>;
+// Layers of variant 2 mix two tile heights inside one launch: the last row block of an expert, when
+// it holds at most 128 rows, goes to a 128 x 256 tile (three stages, loads two slices ahead of the
+// slice being worked on) instead of a 256-row tile whose lower half would multiply rows that do
+// not exist. The blocks keep their 256-row spacing in h1 and y; only the tile that works on them
+// differs. (The K order of every output element is the same in both tiles: same slices, same
+// matrix instruction, so which tile computed a row does not show in its bits.)
+template <typename E, int V>
+using NarrowCfg = Gemm16<E, 128, 256, 2, 4, 64, 3, false, false>;
+template <typename T, int V> constexpr bool kMixedHeights = sizeof(T) == 2 && V == 2 && KLEOS_TUNE_MIXED_HEIGHTS != 0;
+constexpr uint32_t kNarrowTileRows = 128;
 constexpr int kBN = 256;
 constexpr int kGemmThreads = GemmCfg<bf16_t, 0>::kThreads;
+static_assert(NarrowCfg<bf16_t, 2>::kThreads == kGemmThreads, "both tile heights run on the same workgroup");
 static_assert(GemmCfg<bf16_t, 1>::kThreads == kGemmThreads && GemmCfg<bf16_t, 2>::kThreads == kGemmThreads,
               "all variants share the workgroup size");
 constexpr uint32_t kNarrowRows = 128;   // variant 1 when no expert can hold more rows than this
@@ -74,7 +96,9 @@ constexpr int kPhaseThreads = 256;   // gate, slot and combine kernels of the ph
 
 template <typename T, int V>
 constexpr int gemm_smem_bytes() {
-    if constexpr (sizeof(T) == 2) return GemmCfg<T, V>::kSmemBytes;
+    if constexpr (kMixedHeights<T, V>)
+        return GemmCfg<T, V>::kSmemBytes > NarrowCfg<T, V>::kSmemBytes ? GemmCfg<T, V>::kSmemBytes : NarrowCfg<T, V>::kSmemBytes;
+    else if constexpr (sizeof(T) == 2) return GemmCfg<T, V>::kSmemBytes;
     else return gemm_f32_smem_bytes();
 }
 constexpr int kPhasedGemmHeader = 128;
@@ -225,6 +249,7 @@ struct Task {
     uint32_t foreign;   // taken from another XCD's queue: its h1 rows may sit in a different L2
     uint32_t dep;       // down tile: the readiness counter of its row block as seen when handed out
     uint32_t ready;     // down tile whose up-projection row block was already complete when handed out
+    uint32_t narrow;    // the row block holds at most 128 rows and goes to the 128-row tile (layers that mix tile heights)
     uint32_t valid;
 };
 constexpr int kTaskWords = 12;
@@ -235,13 +260,13 @@ __device__ __forceinline__ Task broadcast_task(uint32_t* s_task, const Task& min
     if (threadIdx.x == 0) {
         s_task[0] = mine.e; s_task[1] = mine.kind; s_task[2] = mine.mtile; s_task[3] = mine.ntile;
         s_task[4] = mine.foreign; s_task[5] = mine.ready; s_task[6] = mine.valid; s_task[7] = mine.rows;
-        s_task[8] = mine.dep;
+        s_task[8] = mine.dep; s_task[9] = mine.narrow;
     }
     __syncthreads();
     Task t;
     t.e = s_task[0]; t.kind = s_task[1]; t.mtile = s_task[2]; t.ntile = s_task[3];
     t.foreign = s_task[4]; t.ready = s_task[5]; t.valid = s_task[6]; t.rows = s_task[7];
-    t.dep = s_task[8];
+    t.dep = s_task[8]; t.narrow = s_task[9];
     return t;
 }
 
@@ -272,6 +297,13 @@ __device__ __forceinline__ TileOperands<T> tile_operands(const LayerParams& p, c
         o.c = static_cast<T*>(p.y) + row_base * p.H + col0; o.ldc = p.H; o.act = 2;
     }
     return o;
+}
+
+// Whether row block `mtile` of an expert with `rows` rows goes to the 128-row tile.
+template <typename T, int V>
+__device__ __forceinline__ uint32_t narrow_block(uint32_t rows, uint32_t mtile) {
+    if constexpr (kMixedHeights<T, V>) return uint32_t(rows - mtile * uint32_t(TileShape<T, V>::BM) <= kNarrowTileRows);
+    else return 0u;
 }
 
 // The K slice the tiles of expert e start with, out of k_tiles. Workgroups that run at the same time
@@ -357,7 +389,6 @@ __device__ __forceinline__ void expert_loop(const LayerParams& p, char* smem, ui
     };
 
     if constexpr (sizeof(T) == 2) {
-        using G = GemmCfg<T, V>;
         auto args_of = [&](const Task& t) {
             const TileOperands<T> o = tile_operands<T, V>(p, t);
             GemmTileArgs g;
@@ -365,18 +396,11 @@ __device__ __forceinline__ void expert_loop(const LayerParams& p, char* smem, ui
             g.b_base = reinterpret_cast<const elem16_t*>(o.w); g.bias = reinterpret_cast<const elem16_t*>(o.bias);
             g.c_base = reinterpret_cast<elem16_t*>(o.c);
             g.lda = o.lda; g.ldb = o.K; g.ldc = o.ldc; g.K = o.K; g.m_valid = o.m_valid; g.n_valid = o.n_valid;
-            g.k_first = first_k_slice(t.e, p.E, o.K / uint32_t(G::kSliceK));
+            g.k_first = first_k_slice(t.e, p.E, o.K / uint32_t(GemmCfg<T, V>::kSliceK));
             g.act = o.act;
             return g;
         };
-        typename G::Tile cur_t;
-        typename G::Acc acc;
-        Task cur = next();
-        if (!cur.valid) { flush_stats(); return; }
-        if (cur.kind == 1 && !cur.ready) wait_ready(cur);
-        acquire(cur);
-        int bias_slot = 0;
-        G::begin(cur_t, args_of(cur), 0, bias_slot, smem);
+        static_assert(GemmCfg<T, V>::kSliceK == NarrowCfg<T, V>::kSliceK);
         // An up-projection tile whose stores are issued but which other workgroups have not been told
         // of yet (valid == 0: none). Its stores are known to be complete behind the first barrier of
         // the next tile's main loop, so it is counted from there, at no cost; it is counted at once,
@@ -390,22 +414,49 @@ __device__ __forceinline__ void expert_loop(const LayerParams& p, char* smem, ui
                 pending.valid = 0;
             }
         };
-        for (;;) {
-            G::mainloop(cur_t, acc, smem, [&] { if (pending.valid) publish(pending); });
-            pending.valid = 0;
-            const Task nxt = next();   // its barrier: every wavefront has left the main loop
-            G::finish(cur_t, acc, smem);
-            if (rd.sched && cur.kind == 0) pending = cur;
-            if (!nxt.valid) break;
-            cur = nxt;
-            if (cur.kind == 1 && !cur.ready) {
-                publish_now();   // never wait while holding back a result of our own
-                wait_ready(cur);
-            }
+        // Tiles of one height, from `cur` on, as one pipeline across tiles; returns the first task
+        // that is not of this height (or is not valid), with nothing of its own left unpublished and
+        // every wavefront out of the LDS the tiles used.
+        auto run = [&](auto gemm_tag, auto narrow_tag, Task cur) -> Task {
+            using G = typename decltype(gemm_tag)::type;
+            constexpr uint32_t kNarrow = decltype(narrow_tag)::value ? 1u : 0u;
+            typename G::Tile cur_t;
+            typename G::Acc acc;
+            if (cur.kind == 1 && !cur.ready) wait_ready(cur);
             acquire(cur);
-            G::begin(cur_t, args_of(cur), G::next_stage0(cur_t), bias_slot ^= 1, smem);
+            int bias_slot = 0;
+            G::begin(cur_t, args_of(cur), 0, bias_slot, smem);
+            for (;;) {
+                G::mainloop(cur_t, acc, smem, [&] { if (pending.valid) publish(pending); });
+                pending.valid = 0;
+                const Task nxt = next();   // its barrier: every wavefront has left the main loop
+                G::finish(cur_t, acc, smem);
+                if (rd.sched && cur.kind == 0) pending = cur;
+                if (!nxt.valid || nxt.narrow != kNarrow) {
+                    publish_now();
+                    if (nxt.valid) __syncthreads();   // the other tile height lays the LDS out differently
+                    return nxt;
+                }
+                cur = nxt;
+                if (cur.kind == 1 && !cur.ready) {
+                    publish_now();   // never wait while holding back a result of our own
+                    wait_ready(cur);
+                }
+                acquire(cur);
+                G::begin(cur_t, args_of(cur), G::next_stage0(cur_t), bias_slot ^= 1, smem);
+            }
+        };
+        struct WideTag { using type = GemmCfg<T, V>; };
+        struct NarrowTag { using type = NarrowCfg<T, V>; };
+        Task t = next();
+        while (t.valid) {
+            if constexpr (kMixedHeights<T, V>) {
+                if (t.narrow) t = run(NarrowTag{}, std::true_type{}, t);
+                else t = run(WideTag{}, std::false_type{}, t);
+            } else {
+                t = run(WideTag{}, std::false_type{}, t);
+            }
         }
-        publish_now();
         flush_stats();
     } else {
         for (;;) {
@@ -556,6 +607,7 @@ __global__ __launch_bounds__((TileShape<T, V>::kThreads), (TileShape<T, V>::kPer
                 const uint32_t rows = kept_rows<false>(p, e);
                 if (mtile * TileShape<T, V>::BM >= rows) continue;   // the expert has fewer rows
                 t.e = e; t.rows = rows; t.kind = kind; t.mtile = mtile; t.ntile = rem / tiles_m; t.ready = 1; t.valid = 1;
+                t.narrow = narrow_block<T, V>(rows, mtile);
                 i += gridDim.x;
                 break;
             }
@@ -806,6 +858,7 @@ __global__ __launch_bounds__((TileShape<T, V>::kThreads), (TileShape<T, V>::kPer
         t.mtile = local % s_mt[t.e];
         t.ntile = local / s_mt[t.e];
         t.rows = s_rows[t.e];
+        t.narrow = narrow_block<T, V>(t.rows, t.mtile);
         t.valid = 1;
     };
     auto next = [&]() {

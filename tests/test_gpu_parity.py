@@ -266,6 +266,38 @@ def test_identity_experts_return_input(mode):
     assert rel_fro(moe_out, x) < 1e-6
 
 
+@pytest.mark.parametrize("mode", MODES, ids=MODE_IDS)
+@pytest.mark.parametrize("k", [1, 2])
+def test_tile_heights_mixed_inside_one_layer(mode, k):
+    """A layer whose experts may hold 1024 rows and more walks 256-row blocks, and gives an expert's last
+    block to a 128-row tile when it holds at most 128 rows: experts of 40, 100, 129, 300, 2100 and 403
+    rows (and two without any) in one launch, i.e. blocks of 40 and 100 rows (128-row tile), 129 rows
+    (256-row tile), 256 + 44, 8 x 256 + 52 (full tiles followed by a 128-row tile) and 256 + 147. With
+    k = 2 every token also goes to the next expert, which gives blocks of 140, 229, 173, 96 and 199
+    rows. Token t is sent to its experts by one-hot input features that the gate weights pick up."""
+    S, H, I, E = 3072, 128, 256, 8
+    keys = _keys(S, H, I, E, k, cf=1.0, drop=0)
+    c = moe_ref.cfg_from_keys(keys)
+    assert c.cap_rows >= 1024
+    x, wg, w_up, w_down, b_up, b_down = random_layer(c, seed=91, w_std=0.08, bias_std=0.1)
+    rows = [40, 100, 129, 300, 2100, 403, 0, 0]
+    first = np.repeat(np.arange(E), rows)
+    rng = np.random.default_rng(5)
+    rng.shuffle(first)
+    x[:, :E] = 0.0
+    x[np.arange(S), first] = 8.0
+    x[np.arange(S), (first + 1) % E] = 4.0
+    wg[:, :E] = np.eye(E, dtype=np.float32)
+    wg[:, E:] *= 0.25                                  # the other features only perturb the logits (by about 0.2)
+    iP = pack_inputs(c, x, wg, w_up, w_down, b_up, b_down)
+    d, v, moe_out, err = check_against_oracle(c, keys, iP, mode)
+    expect = np.array(rows)
+    if k == 2:
+        expect = expect + np.roll(expect, 1)
+    np.testing.assert_array_equal(v["expert_count"], expect)
+    assert (v["topk_slot"] >= 0).all()
+
+
 # ------------------------------------------------------------------ back-to-back launches
 @pytest.mark.parametrize("mode", MODES, ids=MODE_IDS)
 def test_experts_that_fill_a_tile_to_every_quarter(mode):
