@@ -53,6 +53,7 @@ SYMBOLS = {
     "kleos_set_device": (C.c_int, []),
     "kleos_get_config": (C.c_int, [C.POINTER(KleosConfigStruct)]),
     "kleos_moe_forward": (C.c_int, [C.c_void_p, C.c_void_p]),
+    "kleos_moe_forward_dense": (C.c_int, [C.c_void_p, C.c_void_p]),
     "kleos_moe_forward_bench": (C.c_int, [C.c_void_p, C.c_void_p, C.c_uint32, C.c_uint32, C.POINTER(C.c_float)]),
     "kleos_moe_forward_static_scratch": (C.c_int, [C.POINTER(KleosConfigStruct), C.c_void_p, C.c_void_p, C.c_void_p]),
     "kleos_static_scratch_prepare": (C.c_int, [C.POINTER(KleosConfigStruct)]),

@@ -31,6 +31,8 @@ struct Context {
     int mode = KLEOS_MODE_FUSED;
     int schedule = KLEOS_SCHEDULE_AUTO;
     size_t zero_begin = 0, zero_end = 0;   // the part of the arena that holds counters (starts as zeros)
+    char* dense_wg = nullptr;       // one expert: zero gate weights and a gate output owned by the library
+    char* dense_gate_out = nullptr;
     float phase_ms[5] = {0, 0, 0, 0, 0};
     double sched_stats[6] = {0, 0, 0, 0, 0, 0};
 };
@@ -52,7 +54,7 @@ size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 struct ArenaLayout {
     size_t logits, topk_expert, topk_prob, combine_den, topk_slot, tile_count, super_count,
-        expert_count, slot_token, h1, y, sched, stamps, tile_prob, super_prob, gate_loss, gate_partial, total;
+        expert_count, slot_token, h1, y, sched, stamps, tile_prob, super_prob, gate_loss, gate_partial, dense_wg, dense_gate_out, total;
     size_t zero_begin, zero_end;   // range that must start as zeros
 };
 
@@ -82,6 +84,10 @@ ArenaLayout layout_arena(const kleos_config_t& c, uint32_t n_tiles, uint32_t n_s
     L.h1 = take(E * R * size_t(c.I) * c.elem_bytes);
     L.y = take(E * R * size_t(c.H) * c.elem_bytes);
     L.gate_partial = take(size_t(gate_splits) * S * c.PX * 4);
+    // one expert: gate weights (zeros) and a gate output of the library's own, for callers that pack the
+    // dense-FFN way, without either (kleos_moe_forward_dense)
+    L.dense_wg = take(E == 1 ? size_t(c.PX) * c.H * c.elem_bytes : 0);
+    L.dense_gate_out = take(E == 1 ? S * size_t(c.PX) * c.elem_bytes : 0);
     L.total = off;
     return L;
 }
@@ -164,11 +170,25 @@ void params_from_arena(LayerParams& p, char* a, const ArenaLayout& L) {
 
 // Enqueues one forward. When ev is non-null (phased mode) it receives 6 recorded events that
 // bracket the five phases.
-int enqueue_forward(Context& c, const void* iP, void* oP, hipEvent_t* ev) {
+int enqueue_forward(Context& c, const void* iP, void* oP, hipEvent_t* ev, bool dense_packing = false) {
     if (!iP || !oP) return fail(KLEOS_EINVAL, "forward: null buffer");
     if ((reinterpret_cast<uintptr_t>(iP) | reinterpret_cast<uintptr_t>(oP)) & 15u)
         return fail(KLEOS_EINVAL, "forward: iP and oP must be 16-byte aligned");
     LayerParams p = bind(c, iP, oP);
+    if (dense_packing) {
+        // iP = A | B1 | B2 | D1 | D2, oP = C (fffn.cuh:43-49): no gate weights, no gate output
+        const kleos_config_t& g = c.cfg;
+        const size_t eb = g.elem_bytes;
+        const char* in = static_cast<const char*>(iP);
+        p.x = in;
+        p.w_up = in + size_t(g.S) * g.H * eb;
+        p.w_down = static_cast<const char*>(p.w_up) + size_t(g.I) * g.H * eb;
+        p.b_up = static_cast<const char*>(p.w_down) + size_t(g.H) * g.I * eb;
+        p.b_down = static_cast<const char*>(p.b_up) + size_t(g.I) * eb;
+        p.wg = c.dense_wg;
+        p.gate_out = c.dense_gate_out;
+        p.moe_out = oP;
+    }
     p.epoch = c.launch_seq++;
     const int dt = int(c.cfg.torch_dtype);
     if (c.mode == KLEOS_MODE_FUSED) {
@@ -417,6 +437,12 @@ extern "C" int kleos_initialize_cfg(const kleos_config_t* user_cfg) {
     KLEOS_HIP_BAIL(hipMemsetAsync(c->arena + L.zero_begin, 0, L.zero_end - L.zero_begin, c->stream));
     KLEOS_HIP_BAIL(hipStreamSynchronize(c->stream));
     params_from_arena(p, c->arena, L);
+    if (cfg.E == 1) {
+        c->dense_wg = c->arena + L.dense_wg;
+        c->dense_gate_out = c->arena + L.dense_gate_out;
+        KLEOS_HIP_BAIL(hipMemsetAsync(c->dense_wg, 0, size_t(cfg.PX) * cfg.H * cfg.elem_bytes, c->stream));
+        KLEOS_HIP_BAIL(hipStreamSynchronize(c->stream));
+    }
     KLEOS_HIP_BAIL(plan_fused(p, int(cfg.torch_dtype), c->num_cus, &c->plan));
     if (c->plan.nwg > kMaxWorkgroups) return bail(fail(KLEOS_EUNSUPPORTED, "persistent grid of %u workgroups exceeds %u", c->plan.nwg, kMaxWorkgroups));
 #undef KLEOS_HIP_BAIL
@@ -512,6 +538,17 @@ extern "C" int kleos_moe_forward(const void* iP, void* oP) {
     if (int rc = require_ctx("kleos_moe_forward")) return rc;
     KLEOS_HIP(hipSetDevice(g_ctx->device));   // moe.cuh:192
     return enqueue_forward(*g_ctx, iP, oP, nullptr);
+}
+
+extern "C" int kleos_moe_forward_dense(const void* iP, void* oP) {
+    if (int rc = require_ctx("kleos_moe_forward_dense")) return rc;
+    Context& c = *g_ctx;
+    if (c.cfg.E != 1) return fail(KLEOS_ESTATE, "kleos_moe_forward_dense: the context holds %u experts; the dense packing is for num_experts 1", c.cfg.E);
+    // the bias block D1 must leave D2 16-byte aligned for the kernels' 16-byte loads
+    if ((size_t(c.cfg.I) * c.cfg.elem_bytes) & 15u)
+        return fail(KLEOS_EUNSUPPORTED, "kleos_moe_forward_dense: intermediate_size * sizeof(Element) must be a multiple of 16");
+    KLEOS_HIP(hipSetDevice(c.device));
+    return enqueue_forward(c, iP, oP, nullptr, true);
 }
 
 extern "C" int kleos_moe_forward_bench(const void* iP, void* oP, uint32_t skip, uint32_t trials,

@@ -213,7 +213,8 @@ struct Gemm16 {
             default: return i == 0 ? L : 0;                                     // all at once
         }
     }
-    static_assert(SPREAD == 0 || (AHEAD2 && (LA + LB) % 8 == 0));
+    static_assert(SPREAD == 0 || !AHEAD2 || (LA + LB) % 8 == 0);
+    static_assert(SPREAD == 0 || AHEAD2 || STAGES >= 3, "one slice ahead, every load is needed at the next barrier");
     static_assert(spread_count(0) + spread_count(1) + spread_count(2) + spread_count(3) == LA + LB);
     static_assert(BK == 32 || BK == 64);
     static_assert(!AHEAD2 || STAGES == 2);
@@ -505,14 +506,21 @@ struct Gemm16 {
                 asm volatile("s_barrier" ::: "memory");
                 if (kt == 0) after_first_barrier();
             };
-            // K step ks carries the loads ks * TN * TM ... of the slice STAGES-1 ahead, one behind each
-            // matrix instruction, until they run out
+            // SPREAD 0: K step ks carries the loads ks * TN * TM ... of the slice STAGES-1 ahead, one behind
+            // each matrix instruction, until they run out (all in the first K step for the tiles in use).
+            // Otherwise the loads are shared out evenly over the K steps of the slice: with three stages
+            // and more they are not needed before the slice after the next one.
             auto ksteps = [&](const char* st, const SliceLoads& l, auto loads_tag) {
                 static_for<kSteps>([&](auto ks_tag) {
                     constexpr int ks = decltype(ks_tag)::value;
-                    constexpr int left = LA + LB - ks * TN * TM;
-                    constexpr int count = !decltype(loads_tag)::value || left <= 0 ? 0 : (left < TN * TM ? left : TN * TM);
-                    kstep(st, ks, l, std::integral_constant<int, ks * TN * TM>{}, std::integral_constant<int, count>{});
+                    constexpr int L = LA + LB;
+                    constexpr int left = L - ks * TN * TM;
+                    constexpr int burst = left <= 0 ? 0 : (left < TN * TM ? left : TN * TM);
+                    constexpr int even = L / kSteps + (ks < L % kSteps ? 1 : 0);
+                    constexpr int even_first = ks * (L / kSteps) + (ks < L % kSteps ? ks : L % kSteps);
+                    constexpr int count = !decltype(loads_tag)::value ? 0 : (SPREAD ? even : burst);
+                    constexpr int first = SPREAD ? even_first : ks * TN * TM;
+                    kstep(st, ks, l, std::integral_constant<int, first>{}, std::integral_constant<int, count>{});
                 });
             };
             const uint32_t ahead = t.k_tiles >= uint32_t(STAGES - 1) ? t.k_tiles - (STAGES - 1) : 0u;   // slices that request a later one

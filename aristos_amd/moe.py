@@ -23,6 +23,12 @@ def forward_host(iP, oP) -> None:
     _capi.check(_capi.lib().kleos_moe_forward(_ptr(iP), _ptr(oP)))
 
 
+def forward_host_dense(iP, oP) -> None:
+    """kleos_moe_forward_dense: num_experts == 1 on the packing of the reference's fffn kernel
+    (fffn.cuh:43-49): iP = x | Wup | Wdown | bup | bdown, oP = moeOut."""
+    _capi.check(_capi.lib().kleos_moe_forward_dense(_ptr(iP), _ptr(oP)))
+
+
 def forward_host_bench(iP, oP, skip: int = 32, trials: int = 32) -> float:
     """kleos::moe::forwardHostBench<skip, trials>(iP, oP, ms) (moe.cuh:146-184): mean milliseconds per
     launch over `trials` launches after `skip` warm-ups. The defaults are the reference driver's

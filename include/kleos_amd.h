@@ -123,10 +123,21 @@ int kleos_get_config(kleos_config_t* cfg);
  * This is the layout the reference's driver packs for any E (csrc/main.cu:23-30). It is NOT the
  * layout the reference's fffn kernel reads, iP = A | B1 | B2 | D1 | D2 and oP = C with no gate
  * blocks (csrc/include/kleos/moe/fffn.cuh:43-49): the reference's driver and its fffn disagree with
- * each other, and this library follows the driver. A caller that packs the fffn way must insert
- * the 64*H gate block (any finite values) and read the result S*64 Elements into oP.
+ * each other. kleos_moe_forward follows the driver; a caller that packs the fffn way calls
+ * kleos_moe_forward_dense instead.
  */
 int kleos_moe_forward(const void* iP, void* oP);
+/*
+ * num_experts == 1 only: the same dense FFN on the packing of the reference's fffn kernel
+ * (csrc/include/kleos/moe/fffn.cuh:43-49, launched by forwardHost at moe.cuh:201-204):
+ * iP: x[S,H] | Wup[I,H] | Wdown[H,I] | bup[I] | bdown[H]   (A | B1 | B2 | D1 | D2; no gate weights)
+ * oP: moeOut[S,H]                                          (C; no gate output)
+ * D2 follows the I entries of D1 (the reference steps over H entries there, fffn.cuh:49, which is the
+ * same place whenever I == H). The gate still runs, on zero gate weights and into a gate output that
+ * the library owns; moeOut has the bits kleos_moe_forward gives for the same operands. Asynchronous on
+ * the library stream. KLEOS_ESTATE when the context holds more than one expert.
+ */
+int kleos_moe_forward_dense(const void* iP, void* oP);
 /*
  * Replaces kleos::moe::forwardHostBench<skip,trials>(iP, oP, ms) (moe.cuh:146-184): `skip` untimed
  * launches, then `trials` launches bracketed by events on the library stream; *ms_per_launch is the

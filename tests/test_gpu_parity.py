@@ -298,6 +298,46 @@ def test_tile_heights_mixed_inside_one_layer(mode, k):
     assert (v["topk_slot"] >= 0).all()
 
 
+@pytest.mark.parametrize("dt", [2, 0])
+def test_dense_packing_of_a_single_expert(dt):
+    """num_experts == 1 on the packing the reference's fffn kernel reads (fffn.cuh:43-49): iP = x | Wup |
+    Wdown | bup | bdown with no gate weights, oP = moeOut with no gate output. kleos_moe_forward_dense
+    gives the bits kleos_moe_forward gives on the driver's packing of the same operands (which the
+    other tests check against the oracle), and refuses a context with more than one expert."""
+    S, H, I = 256, 128, 192                            # I != H: the second bias vector follows I entries
+    keys = _keys(S, H, I, 1, 1, dt=dt)
+    c = moe_ref.cfg_from_keys(keys)
+    x, wg, w_up, w_down, b_up, b_down = random_layer(c, seed=57, w_std=0.08, bias_std=0.1)
+    iP_np = pack_inputs(c, x, wg, w_up, w_down, b_up, b_down)
+    check_against_oracle(c, keys, iP_np, ka.MODE_FUSED)
+    # the same operands without the 64 x H gate block: everything behind x moves up
+    dense_np = np.concatenate([iP_np[:S * H], iP_np[S * H + c.PX * H:]])
+    assert dense_np.size == S * H + 2 * I * H + I + H
+    d = ka.initialize(keys)
+    try:
+        oP = synth.alloc_outputs(d)
+        ka.moe.forward_host(_to_device(c, iP_np), oP)
+        ka.moe.stream_synchronize()
+        want = _out_to_np(c, oP)[S * c.PX:].copy()
+        dense_out = torch.full((S * H,), float("nan"), dtype=oP.dtype, device="cuda")
+        for mode in (ka.MODE_FUSED, ka.MODE_PHASED):
+            ka.moe.set_mode(mode)
+            dense_out.fill_(float("nan"))
+            torch.cuda.synchronize()
+            ka.moe.forward_host_dense(_to_device(c, dense_np), dense_out)
+            ka.moe.stream_synchronize()
+            np.testing.assert_array_equal(_out_to_np(c, dense_out), want)
+    finally:
+        ka.finalize()
+    d = ka.initialize(_keys(S, H, I, 4, 1, dt=dt))
+    try:
+        with pytest.raises(ka.KleosError) as ei:
+            ka.moe.forward_host_dense(16, 16)
+        assert ei.value.code == ka._capi.KLEOS_ESTATE
+    finally:
+        ka.finalize()
+
+
 # ------------------------------------------------------------------ back-to-back launches
 @pytest.mark.parametrize("mode", MODES, ids=MODE_IDS)
 def test_experts_that_fill_a_tile_to_every_quarter(mode):
