@@ -20,7 +20,7 @@ HIPCC_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wextra", "-Wno-unused-parameter", "-Wno-pass-failed",
 ]
-SOURCES = ["config.cpp", "capi.hip", "kernels.hip", "kernels_f32.hip", "kernels_bf16.hip", "kernels_f16.hip"]
+SOURCES = ["config.cpp", "capi.hip", "kernels.hip", "kernels_f32.hip", "kernels_tf32.hip", "kernels_bf16.hip", "kernels_f16.hip"]
 
 
 def _hipcc() -> str:

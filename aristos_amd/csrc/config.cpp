@@ -183,9 +183,6 @@ extern "C" int kleos_config_derive(kleos_config_t* c) {
     if (c->is_training > 1) return fail(KLEOS_EINVAL, "is_training must be 0 or 1, got %u", c->is_training);
     if (c->hidden_act > KLEOS_ACT_GELU) return fail(KLEOS_EINVAL, "hidden_act must be 0 (relu) or 1 (gelu), got %u", c->hidden_act);
     if (c->torch_dtype > KLEOS_DTYPE_FP16) return fail(KLEOS_EINVAL, "torch_dtype must be 0..3, got %u", c->torch_dtype);
-    if (c->torch_dtype == KLEOS_DTYPE_TF32)
-        return fail(KLEOS_EUNSUPPORTED, "torch_dtype 1 (tf32, the value the reference ships in kleos_config.json) is unsupported: CDNA4 has no "
-                    "tf32 matrix path; set \"torch_dtype\" to 2 (bf16), 3 (fp16) or 0 (fp32) in the configuration");
     if (c->num_experts < 1) return fail(KLEOS_EINVAL, "num_experts must be >= 1");
     if (c->num_experts > 65535) return fail(KLEOS_EINVAL, "num_experts must be <= 65535 (types.cuh:479), got %u", c->num_experts);
     if (c->expert_top_k < 1) return fail(KLEOS_EINVAL, "expert_top_k must be >= 1");
@@ -216,7 +213,7 @@ extern "C" int kleos_config_derive(kleos_config_t* c) {
     c->EC = uint32_t(ec);
     c->pEC = uint32_t(ceil_div(c->EC, 128) * 128);                                      // types.cuh:500
     c->cap_rows = uint32_t(std::min<uint64_t>(c->pEC, S));
-    c->elem_bytes = (c->torch_dtype == KLEOS_DTYPE_FP32) ? 4u : 2u;
+    c->elem_bytes = (c->torch_dtype == KLEOS_DTYPE_FP32 || c->torch_dtype == KLEOS_DTYPE_TF32) ? 4u : 2u;
     // Packed buffers: moe.cuh:92-98, main.cu:23-30.
     const uint64_t H = c->H, I = c->I, E = c->E, PX = c->PX;
     c->off_x = 0;

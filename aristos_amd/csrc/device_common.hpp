@@ -22,7 +22,26 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 constexpr int kWave = 64;
 
+// tf32 (torch_dtype 1, the reference's cute::tfloat32_t, csrc/include/kleos/types.cuh:128-131): an
+// Element stored in 32 bits of which the matrix cores of the reference's hardware read the sign,
+// the exponent and the upper 10 mantissa bits. CDNA4 has no tf32 matrix instruction: the fp32
+// matrix instructions run on operands whose lower 13 mantissa bits are cleared (products of two
+// such values are exact in fp32, as they are in a tf32 tensor core), and every Element the layer
+// produces is rounded to 10 mantissa bits, ties to even, with the lower bits cleared
+// (cutlass::NumericConverter<tfloat32_t, float> rounds the same way and leaves the lower bits
+// undefined).
+struct tf32_t { float v; };
+__device__ __forceinline__ float tf32_operand(float v) {
+    return __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, v) & 0xffffe000u);
+}
+__device__ __forceinline__ float tf32_round(float v) {
+    uint32_t u = __builtin_bit_cast(uint32_t, v);
+    if ((u & 0x7f800000u) != 0x7f800000u) u += 0x0fffu + ((u >> 13) & 1u);   // infinities and NaNs keep their bits
+    return __builtin_bit_cast(float, u & 0xffffe000u);
+}
+
 __device__ __forceinline__ float elem_to_float(bf16_t v) { return static_cast<float>(v); }
+__device__ __forceinline__ float elem_to_float(tf32_t v) { return v.v; }   // as stored (a bias, a gate output)
 __device__ __forceinline__ float elem_to_float(f16_t v) { return static_cast<float>(v); }
 __device__ __forceinline__ float elem_to_float(float v) { return v; }
 
@@ -31,6 +50,8 @@ template <typename T>
 __device__ __forceinline__ T float_to_elem(float v);
 template <>
 __device__ __forceinline__ float float_to_elem<float>(float v) { return v; }
+template <>
+__device__ __forceinline__ tf32_t float_to_elem<tf32_t>(float v) { return tf32_t{tf32_round(v)}; }
 template <>
 __device__ __forceinline__ bf16_t float_to_elem<bf16_t>(float v) { return static_cast<bf16_t>(v); }
 template <>
@@ -85,6 +106,12 @@ __device__ __forceinline__ f32x4 mma16_step(u32x4 a, u32x4 b, f32x4 acc, float) 
     acc = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[2], fb[2], acc, 0, 0, 0);
     acc = __builtin_amdgcn_mfma_f32_16x16x4f32(fa[3], fb[3], acc, 0, 0, 0);
     return acc;
+}
+
+// tf32: the same fp32 instructions on operands cut to their upper 10 mantissa bits.
+__device__ __forceinline__ f32x4 mma16_step(u32x4 a, u32x4 b, f32x4 acc, tf32_t) {
+    const u32x4 mask{0xffffe000u, 0xffffe000u, 0xffffe000u, 0xffffe000u};
+    return mma16_step(a & mask, b & mask, acc, float{});
 }
 
 // The value another lane of the same row of 16 lanes holds, by the lane selects of the vector ALU

@@ -199,22 +199,17 @@ struct Gemm16 {
     static constexpr int kSteps = BK / 16;                         // matrix instructions consume 16 values of K
     static constexpr int kPanelRows = kEpiloguePanelRows;          // epilogue staging: 32 rows x 64 columns per wavefront
     // loads of a slice (per wavefront) issued at the last K step of the slice two before it [0] and at
-    // K steps 0, 1, 2 of the slice before it [1..3]; SPREAD >= 10: weight rows before activation rows
-    static constexpr int kPolicy = SPREAD % 10;
-    static constexpr bool kWeightsFirst = SPREAD >= 10;
+    // K steps 0, 1, 2 of the slice before it [1..3]
     static constexpr int spread_count(int i) {
         constexpr int L = LA + LB;
-        switch (kPolicy) {
-            case 1: return i < 2 ? L / 2 : 0;                                   // 4 4 0 0
+        switch (SPREAD) {
+            case 1: return i < 2 ? L / 2 : 0;                                                       // 4 4 0 0
             case 2: return i == 0 || i == 1 ? (3 * L) / 8 : (i == 2 ? L - 2 * ((3 * L) / 8) : 0);   // 3 3 2 0
-            case 3: return L / 4;                                               // 2 2 2 2
-            case 4: return i == 0 ? L / 2 : (i < 3 ? L / 4 : 0);                // 4 2 2 0
-            case 5: return i == 0 ? L / 4 : (i < 3 ? (3 * L) / 8 : 0);          // 2 3 3 0
-            default: return i == 0 ? L : 0;                                     // all at once
+            default: return i == 0 ? L : 0;                                                         // all at once
         }
     }
-    static_assert(SPREAD == 0 || !AHEAD2 || (LA + LB) % 8 == 0);
-    static_assert(SPREAD == 0 || AHEAD2 || STAGES >= 3, "one slice ahead, every load is needed at the next barrier");
+    static_assert(SPREAD >= 0 && SPREAD <= 2);
+    static_assert(SPREAD == 0 || (AHEAD2 && (LA + LB) % 8 == 0));
     static_assert(spread_count(0) + spread_count(1) + spread_count(2) + spread_count(3) == LA + LB);
     static_assert(BK == 32 || BK == 64);
     static_assert(!AHEAD2 || STAGES == 2);
@@ -262,16 +257,15 @@ struct Gemm16 {
                                              STREAM_B ? kNonTemporal : 0);
     }
 
-    // Load number j (0 <= j < LA + LB) of K slice kt in the order the policy issues them.
+    // Load number j (0 <= j < LA + LB) of a K slice: activation rows first (they come from L2 and return
+    // early), then the weight rows.
     static __device__ __forceinline__ void issue_one(const Tile& t, char* sa, char* sb, uint32_t k0, int j) {
         const int wave = threadIdx.x >> 6;
-        const bool is_w = kWeightsFirst ? j < LB : j >= LA;
-        const int i = kWeightsFirst ? (j < LB ? j : j - LB) : (j < LA ? j : j - LA);
-        if (is_w)
-            __builtin_amdgcn_global_load_lds((global_cptr)(t.pb[i] + k0), (lds_ptr)(sb + 1024 * (wave + kWaves * i)), 16, 0,
+        if (j >= LA)
+            __builtin_amdgcn_global_load_lds((global_cptr)(t.pb[j - LA] + k0), (lds_ptr)(sb + 1024 * (wave + kWaves * (j - LA))), 16, 0,
                                              STREAM_B ? kNonTemporal : 0);
         else
-            __builtin_amdgcn_global_load_lds((global_cptr)(t.pa[i] + k0), (lds_ptr)(sa + 1024 * (wave + kWaves * i)), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((global_cptr)(t.pa[j] + k0), (lds_ptr)(sa + 1024 * (wave + kWaves * j)), 16, 0, 0);
     }
     // Loads first .. first + count - 1 of K slice kt.
     template <int FIRST, int COUNT>
@@ -436,18 +430,7 @@ struct Gemm16 {
                     else if (i < TN + TM) fx[nb][i - TN] = __builtin_bit_cast(vec8, load16(st + (base_x ^ ((ks + 1) << 5)) + (i - TN) * 32 * kRowBytes));
                 }
                 if constexpr (COUNT > 0) {
-                    if (i % kEvery == 0 && i / kEvery < COUNT) {
-                        if constexpr (AHEAD2) {
-                            issue_one(t, l.sa, l.sb, l.k0, FIRST + i / kEvery);
-                        } else {
-                            const int li = FIRST + i / kEvery;
-                            if (li < LA)
-                                __builtin_amdgcn_global_load_lds((global_cptr)(t.pa[li] + l.k0), (lds_ptr)(l.sa + 1024 * (wave + kWaves * li)), 16, 0, 0);
-                            else if (li < LA + LB)
-                                __builtin_amdgcn_global_load_lds((global_cptr)(t.pb[li - LA] + l.k0), (lds_ptr)(l.sb + 1024 * (wave + kWaves * (li - LA))), 16,
-                                                                 0, STREAM_B ? kNonTemporal : 0);
-                        }
-                    }
+                    if (i % kEvery == 0 && i / kEvery < COUNT) issue_one(t, l.sa, l.sb, l.k0, FIRST + i / kEvery);
                 }
             }
             __builtin_amdgcn_sched_barrier(0);
@@ -506,21 +489,16 @@ struct Gemm16 {
                 asm volatile("s_barrier" ::: "memory");
                 if (kt == 0) after_first_barrier();
             };
-            // SPREAD 0: K step ks carries the loads ks * TN * TM ... of the slice STAGES-1 ahead, one behind
-            // each matrix instruction, until they run out (all in the first K step for the tiles in use).
-            // Otherwise the loads are shared out evenly over the K steps of the slice: with three stages
-            // and more they are not needed before the slice after the next one.
+            // K step ks carries the loads ks * TN * TM ... of the slice STAGES-1 ahead, one behind each
+            // matrix instruction, until they run out (sharing them out evenly over the four K steps,
+            // which three stages would allow, changes nothing where it was measured: 2.93 against
+            // 2.92 ms per forward at the 256-expert top-8 shape, which is bound by HBM)
             auto ksteps = [&](const char* st, const SliceLoads& l, auto loads_tag) {
                 static_for<kSteps>([&](auto ks_tag) {
                     constexpr int ks = decltype(ks_tag)::value;
-                    constexpr int L = LA + LB;
-                    constexpr int left = L - ks * TN * TM;
-                    constexpr int burst = left <= 0 ? 0 : (left < TN * TM ? left : TN * TM);
-                    constexpr int even = L / kSteps + (ks < L % kSteps ? 1 : 0);
-                    constexpr int even_first = ks * (L / kSteps) + (ks < L % kSteps ? ks : L % kSteps);
-                    constexpr int count = !decltype(loads_tag)::value ? 0 : (SPREAD ? even : burst);
-                    constexpr int first = SPREAD ? even_first : ks * TN * TM;
-                    kstep(st, ks, l, std::integral_constant<int, first>{}, std::integral_constant<int, count>{});
+                    constexpr int left = LA + LB - ks * TN * TM;
+                    constexpr int count = !decltype(loads_tag)::value || left <= 0 ? 0 : (left < TN * TM ? left : TN * TM);
+                    kstep(st, ks, l, std::integral_constant<int, ks * TN * TM>{}, std::integral_constant<int, count>{});
                 });
             };
             const uint32_t ahead = t.k_tiles >= uint32_t(STAGES - 1) ? t.k_tiles - (STAGES - 1) : 0u;   // slices that request a later one
@@ -607,13 +585,23 @@ struct Gemm16 {
 constexpr int kF32Tile = 64, kF32BK = 16, kF32Pad = 68;
 constexpr int gemm_f32_smem_bytes() { return 2 * kF32BK * kF32Pad * 4; }
 
-template <int ACT>
+// T: float, or tf32_t - then the operands lose their lower 13 mantissa bits on the way into LDS
+// and the results are rounded to tf32 Elements.
+template <int ACT, typename T>
 __device__ __forceinline__ void gemm_tile_f32(
-    const float* __restrict__ a_base, const int32_t* __restrict__ a_row_index, uint32_t a_rows, uint32_t lda,
+    const T* __restrict__ a_elems, const int32_t* __restrict__ a_row_index, uint32_t a_rows, uint32_t lda,
     uint32_t m_valid,
-    const float* __restrict__ b_base, uint32_t ldb, uint32_t n_valid,
-    const float* __restrict__ bias, float* __restrict__ c_base, uint32_t ldc, uint32_t K,
+    const T* __restrict__ b_elems, uint32_t ldb, uint32_t n_valid,
+    const T* __restrict__ bias_elems, T* __restrict__ c_elems, uint32_t ldc, uint32_t K,
     char* smem) {
+    static_assert(sizeof(T) == 4);
+    constexpr bool kTf32 = std::is_same<T, tf32_t>::value;
+    const float* a_base = reinterpret_cast<const float*>(a_elems);
+    const float* b_base = reinterpret_cast<const float*>(b_elems);
+    const float* bias = reinterpret_cast<const float*>(bias_elems);
+    float* c_base = reinterpret_cast<float*>(c_elems);
+    auto operand = [](float v) { return kTf32 ? tf32_operand(v) : v; };
+    auto result = [](float v) { return kTf32 ? tf32_round(v) : v; };
     float (*As)[kF32Pad] = reinterpret_cast<float (*)[kF32Pad]>(smem);
     float (*Bs)[kF32Pad] = reinterpret_cast<float (*)[kF32Pad]>(smem + kF32BK * kF32Pad * 4);
     const int tid = threadIdx.x;
@@ -644,8 +632,8 @@ __device__ __forceinline__ void gemm_tile_f32(
         __syncthreads();
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            As[ld_kq * 4 + j][ld_row] = va[j];
-            Bs[ld_kq * 4 + j][ld_row] = vb[j];
+            As[ld_kq * 4 + j][ld_row] = operand(va[j]);
+            Bs[ld_kq * 4 + j][ld_row] = operand(vb[j]);
         }
         __syncthreads();
 #pragma unroll
@@ -667,12 +655,12 @@ __device__ __forceinline__ void gemm_tile_f32(
             if (n0 + 4 <= n_valid && ((reinterpret_cast<uintptr_t>(dst) & 15u) == 0)) {
                 f32x4 o;
 #pragma unroll
-                for (int j = 0; j < 4; ++j) o[j] = activate<ACT>(acc[4 * q + j] + bias[n0 + j]);
+                for (int j = 0; j < 4; ++j) o[j] = result(activate<ACT>(acc[4 * q + j] + bias[n0 + j]));
                 store16_through(dst, __builtin_bit_cast(u32x4, o));
             } else {
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
-                    if (n0 + j < n_valid) store_through(dst + j, activate<ACT>(acc[4 * q + j] + bias[n0 + j]));
+                    if (n0 + j < n_valid) store_through(dst + j, result(activate<ACT>(acc[4 * q + j] + bias[n0 + j])));
             }
         }
     }

@@ -7,6 +7,7 @@
 namespace kleos_amd {
 
 KLEOS_EXTERN_ELEMENT(float)
+KLEOS_EXTERN_ELEMENT(tf32_t)
 KLEOS_EXTERN_ELEMENT(bf16_t)
 KLEOS_EXTERN_ELEMENT(f16_t)
 
@@ -47,10 +48,11 @@ uint32_t gate_splits_for(uint32_t S, uint32_t H, uint32_t E, uint32_t PX, int dt
     return splits < 1 ? 1u : splits;
 }
 
-// Calls go(Element{}) for the Element type of a torch_dtype value (kleos_amd.h: 0 fp32, 2 bf16, 3 fp16).
+// Calls go(Element{}) for the Element type of a torch_dtype value (kleos_amd.h: 0 fp32, 1 tf32, 2 bf16, 3 fp16).
 template <typename F>
 hipError_t dispatch_dtype(int dtype, F&& go) {
     switch (dtype) {
+        case 1: return go(tf32_t{});
         case 2: return go(bf16_t{});
         case 3: return go(f16_t{});
         default: return go(float{});

@@ -60,15 +60,12 @@ constexpr int kXcds = 8;
 #ifndef KLEOS_TUNE_V2_SPREAD
 #define KLEOS_TUNE_V2_SPREAD 1       // variant 2: two slices ahead, 4 + 4 over two K steps; -1: one slice ahead
 #endif
-#ifndef KLEOS_TUNE_V1_SPREAD
-#define KLEOS_TUNE_V1_SPREAD 0       // variant 1 (three stages): 1 = loads of a slice shared out over its four K steps (no gain measured)
-#endif
 #ifndef KLEOS_TUNE_MIXED_HEIGHTS
 #define KLEOS_TUNE_MIXED_HEIGHTS 1   // variant 2: 128-row tiles for last row blocks of at most 128 rows
 #endif
 template <typename E, int V>
 using GemmCfg = std::conditional_t<V == 0, Gemm16<E, 256, 256, 4, 2, 64, 2, true, true, KLEOS_TUNE_V0_SPREAD>,
-                std::conditional_t<V == 1, Gemm16<E, 128, 256, 2, 4, 64, 3, true, false, KLEOS_TUNE_V1_SPREAD>,
+                std::conditional_t<V == 1, Gemm16<E, 128, 256, 2, 4, 64, 3, true, false>,
                                    Gemm16<E, 256, 256, 2, 4, 64, 2, false, (KLEOS_TUNE_V2_SPREAD >= 0), (KLEOS_TUNE_V2_SPREAD >= 0 ? KLEOS_TUNE_V2_SPREAD : 0)>>>;
 // Layers of variant 2 mix two tile heights inside one launch: the last row block of an expert, when
 // it holds at most 128 rows, goes to a 128 x 256 tile (three stages, loads two slices ahead of the
@@ -95,6 +92,7 @@ template <typename T, int V = 0> struct TileShape {
     static constexpr int BM = V == 1 ? 128 : 256, BN = kBN, kThreads = kGemmThreads, kPerCu = 1;
 };
 template <int V> struct TileShape<float, V> { static constexpr int BM = kF32Tile, BN = kF32Tile, kThreads = 256, kPerCu = 1; };
+template <int V> struct TileShape<tf32_t, V> : TileShape<float, V> {};
 constexpr int kPhaseThreads = 256;   // gate, slot and combine kernels of the phased mode
 
 template <typename T, int V>

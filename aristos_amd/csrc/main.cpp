@@ -50,6 +50,16 @@ uint16_t to_bf16(float v) {
     return uint16_t(u >> 16);
 }
 
+// fp32 -> tf32 held in 32 bits: 10 mantissa bits, round to nearest even, the lower 13 bits cleared.
+float to_tf32(float v) {
+    uint32_t u;
+    std::memcpy(&u, &v, 4);
+    if ((u & 0x7f800000u) != 0x7f800000u) u += 0x0fffu + ((u >> 13) & 1u);
+    u &= 0xffffe000u;
+    std::memcpy(&v, &u, 4);
+    return v;
+}
+
 // fp32 -> IEEE binary16 bits, round to nearest even; overflow to infinity, gradual underflow.
 uint16_t to_f16(float v) {
     uint32_t u;
@@ -107,6 +117,8 @@ int main(int argc, char** argv) {
         for (uint64_t i = 0; i < dZ; ++i) elems[i] = f16 ? to_f16(host[i]) : to_bf16(host[i]);   // main.cu:59-62
         HIP_OK(hipMemcpy(p, elems.data(), dZ * 2, hipMemcpyHostToDevice));
     } else {
+        if (c.torch_dtype == KLEOS_DTYPE_TF32)
+            for (uint64_t i = 0; i < dZ; ++i) host[i] = to_tf32(host[i]);   // main.cu:59-62, Element = tfloat32_t
         HIP_OK(hipMemcpy(p, host.data(), dZ * 4, hipMemcpyHostToDevice));
     }
     float timed = 0;

@@ -136,7 +136,17 @@ def make_inputs(workload: Workload, seed: int = 0, device: str = "cuda", portabl
 
     if workload.zipf_s > 0:
         _inject_zipf_bias(buf, d, workload, seed)
+    if d.keys.torch_dtype == 1:
+        _round_tf32_(buf)   # main.cu:59-62 converts every input to Element, here tfloat32_t
     return buf, d
+
+
+def _round_tf32_(buf) -> None:
+    """In place: fp32 values to tf32 held in 32 bits (10 mantissa bits, ties to even, lower bits cleared)."""
+    import torch
+    u = buf.view(torch.int32)
+    finite = (u & 0x7F800000) != 0x7F800000
+    u.copy_(torch.where(finite, u + 0x0FFF + ((u >> 13) & 1), u) & ~0x1FFF)
 
 
 def _inject_zipf_bias(buf, d: DerivedConfig, w: Workload, seed: int) -> float:

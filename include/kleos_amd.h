@@ -33,7 +33,13 @@ enum {
 };
 
 /* ---- configuration -------------------------------------------------------------------------- */
-/* torch_dtype enumeration of the reference (csrc/kleos_config.schema.json:64-68). */
+/* torch_dtype enumeration of the reference (csrc/kleos_config.schema.json:64-68). tf32 (the value the
+ * reference ships, csrc/kleos_config.json:15) is an Element stored in 32 bits whose matrix products
+ * use 10 mantissa bits of each operand (csrc/include/kleos/types.cuh:128-131, cute::tfloat32_t). CDNA4
+ * has no tf32 matrix instruction: the products run on the fp32 matrix instructions with the lower 13
+ * mantissa bits of the operands cleared, which gives the products a tf32 tensor core gives, and every
+ * Element the layer writes (gateOut, moeOut, the activations between the projections) is fp32 rounded
+ * to 10 mantissa bits, ties to even, lower bits zero. Buffers are packed as for fp32. */
 enum { KLEOS_DTYPE_FP32 = 0, KLEOS_DTYPE_TF32 = 1, KLEOS_DTYPE_BF16 = 2, KLEOS_DTYPE_FP16 = 3 };
 /* hidden_act enumeration of the reference (csrc/kleos_config.schema.json:29-33). */
 enum { KLEOS_ACT_RELU = 0, KLEOS_ACT_GELU = 1 };
@@ -86,7 +92,7 @@ int kleos_config_parse_file(const char* path, kleos_config_t* cfg);
 void kleos_config_defaults(kleos_config_t* cfg);
 /* Validate the keys and fill the derived fields. Enforces the reference's static_asserts
  * (csrc/include/kleos/bootstrap.cuh:542-545; types.cuh:479,496-497): S % 128 == 0, I % 64 == 0,
- * H % 64 == 0, k <= E, E <= 65535, capacity_factor >= 1. tf32 yields KLEOS_EUNSUPPORTED. */
+ * H % 64 == 0, k <= E, E <= 65535, capacity_factor >= 1. */
 int kleos_config_derive(kleos_config_t* cfg);
 
 /* ---- lifecycle ------------------------------------------------------------------------------ */
@@ -94,7 +100,7 @@ int kleos_config_derive(kleos_config_t* cfg);
  * selects the device, creates the library stream and allocates every scratch arena (routing
  * tables, intermediate activations, scheduler counters) the forward needs, as the reference's
  * Bookkeeping arenas are (bootstrap.cuh:377-391). Fails with KLEOS_ESTATE "Already Initialized",
- * and with KLEOS_EUNSUPPORTED for what this build leaves out: tf32, more than 512 experts, top-k
+ * and with KLEOS_EUNSUPPORTED for what this build leaves out: more than 512 experts, top-k
  * above 32 together with more than 256 experts. */
 int kleos_initialize(const char* config_json_path);
 int kleos_initialize_cfg(const kleos_config_t* cfg);

@@ -38,6 +38,10 @@
  *     Element atomicAdd in arrival order, processor.cuh:157,165);
  *   - a k=1 token whose expert dropped it yields a zero row (the reference leaves the row
  *     unwritten).
+ *   - tf32 (torch_dtype 1): the conversion is CUTLASS's (absent third-party code, restated; see
+ *     moe_ref_round_tf32), pinned against an independent frexp/rint/ldexp rounding and crafted ties;
+ *     that a tf32 tensor core ignores the lower 13 operand bits is the hardware's documented
+ *     behaviour, which no file of the reference states: parity unpinned for that choice;
  *   Functions whose exact bits only a run of the reference could fix (fast-math exp/div ULPs,
  *   atomic order) are "parity unpinned" at the bit level and are compared within tolerance.
  */
@@ -108,8 +112,30 @@ float moe_ref_f16_bits_to_f32(uint16_t b) {
 }
 float moe_ref_round_f16(float v) { return moe_ref_f16_bits_to_f32(moe_ref_f32_to_f16_bits(v)); }
 
+/* tf32 (torch_dtype 1; the reference's cute::tfloat32_t, types.cuh:128-131): an Element held in 32
+ * bits. Conversion from fp32 is cutlass::NumericConverter<tfloat32_t, float> of CUTLASS (a dependency
+ * the reference fetches at its main branch, csrc/CMakeLists.txt:106-167, absent here; restated from its
+ * published source): round to nearest, ties to even, at mantissa bit 13, infinities and NaNs
+ * untouched. CUTLASS leaves the 13 lower bits undefined; they are cleared here. A tensor core reads
+ * only the upper 19 bits of a tf32 operand: moe_ref_tf32_operand. */
+float moe_ref_round_tf32(float v) {
+    uint32_t u;
+    memcpy(&u, &v, 4);
+    if ((u & 0x7f800000u) != 0x7f800000u) u += 0x0fffu + ((u >> 13) & 1u);
+    u &= 0xffffe000u;
+    memcpy(&v, &u, 4);
+    return v;
+}
+float moe_ref_tf32_operand(float v) {
+    uint32_t u;
+    memcpy(&u, &v, 4);
+    u &= 0xffffe000u;
+    memcpy(&v, &u, 4);
+    return v;
+}
+
 static inline float to_elem(float v, uint32_t dtype) {
-    return dtype == 2 ? moe_ref_round_bf16(v) : dtype == 3 ? moe_ref_round_f16(v) : v;
+    return dtype == 2 ? moe_ref_round_bf16(v) : dtype == 3 ? moe_ref_round_f16(v) : dtype == 1 ? moe_ref_round_tf32(v) : v;
 }
 
 /* Packed-buffer element i as fp32. */
@@ -120,6 +146,7 @@ static inline float load_elem(const void* p, size_t i, uint32_t dtype) {
 static inline void store_elem(void* p, size_t i, float v, uint32_t dtype) {
     if (dtype == 2) ((uint16_t*)p)[i] = moe_ref_f32_to_bf16_bits(v);
     else if (dtype == 3) ((uint16_t*)p)[i] = moe_ref_f32_to_f16_bits(v);
+    else if (dtype == 1) ((float*)p)[i] = moe_ref_round_tf32(v);
     else ((float*)p)[i] = v;
 }
 static void load_elems(const void* p, size_t off, size_t n, uint32_t dtype, float* dst) {
@@ -129,6 +156,10 @@ static void load_elems(const void* p, size_t off, size_t n, uint32_t dtype, floa
     } else if (dtype == 3) {
         const uint16_t* s = (const uint16_t*)p + off;
         for (size_t i = 0; i < n; ++i) dst[i] = moe_ref_f16_bits_to_f32(s[i]);
+    } else if (dtype == 1) {
+        /* rows that feed a matrix product: what a tf32 tensor core reads of them */
+        const float* s = (const float*)p + off;
+        for (size_t i = 0; i < n; ++i) dst[i] = moe_ref_tf32_operand(s[i]);
     } else {
         memcpy(dst, (const float*)p + off, n * sizeof(float));
     }
@@ -165,7 +196,7 @@ int moe_ref_threads(void) {
 int moe_ref_derive(moe_ref_cfg* c) {
     if (!c || !c->S || !c->H || !c->I || !c->E || !c->k || c->k > c->E) return -1;
     if (c->S % 128 || c->H % 64 || c->I % 64 || !(c->capacity_factor >= 1.0)) return -1;
-    if (c->dtype != 0 && c->dtype != 2 && c->dtype != 3) return -1;
+    if (c->dtype > 3) return -1;
     c->PX = (c->E + 63u) / 64u * 64u;                                   /* types.cuh:481 */
     double base = c->drop_tokens ? (double)((c->S + c->E - 1u) / c->E) : (double)c->S;
     c->EC = (uint32_t)ceil(base * c->capacity_factor * (double)c->k - 1e-9); /* types.cuh:498-499 */

@@ -34,6 +34,10 @@ float moe_ref_bf16_bits_to_f32(uint16_t b);
 float moe_ref_round_f16(float v);
 uint16_t moe_ref_f32_to_f16_bits(float v);
 float moe_ref_f16_bits_to_f32(uint16_t b);
+/* tf32 held in 32 bits: fp32 rounded to 10 mantissa bits (ties to even, lower 13 bits cleared), and
+ * what a tensor core reads of a 32-bit operand (lower 13 bits cleared, no rounding). */
+float moe_ref_round_tf32(float v);
+float moe_ref_tf32_operand(float v);
 
 /* logits[t,e] = sum_h x[t,h] * wg[e,h], fp32 accumulation. x [S,H], wg [E,H], logits [S,E]. */
 void moe_ref_gate_logits(uint32_t S, uint32_t H, uint32_t E, const float* x, const float* wg,

@@ -55,6 +55,10 @@ def lib() -> C.CDLL:
         h.moe_ref_round_bf16.argtypes = [C.c_float]
         h.moe_ref_round_f16.restype = C.c_float
         h.moe_ref_round_f16.argtypes = [C.c_float]
+        h.moe_ref_round_tf32.restype = C.c_float
+        h.moe_ref_round_tf32.argtypes = [C.c_float]
+        h.moe_ref_tf32_operand.restype = C.c_float
+        h.moe_ref_tf32_operand.argtypes = [C.c_float]
         h.moe_ref_f32_to_f16_bits.restype = C.c_uint16
         h.moe_ref_f32_to_f16_bits.argtypes = [C.c_float]
         h.moe_ref_f16_bits_to_f32.restype = C.c_float
@@ -118,8 +122,19 @@ def f32_to_bf16_bits(a: np.ndarray) -> np.ndarray:
     return (rounded >> 16).astype(np.uint16)
 
 
+def round_tf32(a: np.ndarray) -> np.ndarray:
+    """fp32 -> tf32 held in 32 bits: 10 mantissa bits, ties to even, the lower 13 bits cleared."""
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    u = a.view(np.uint32).astype(np.uint64)
+    finite = (u & 0x7F800000) != 0x7F800000
+    r = np.where(finite, u + 0x0FFF + ((u >> 13) & 1), u) & 0xFFFFE000
+    return r.astype(np.uint32).view(np.float32).reshape(a.shape)
+
+
 def f32_to_elem_bits(a: np.ndarray, c: RefCfg) -> np.ndarray:
     """fp32 values -> the packed Element representation of the configuration."""
+    if c.dtype == 1:
+        return round_tf32(a)
     if c.dtype == 2:
         return f32_to_bf16_bits(a)
     if c.dtype == 3:

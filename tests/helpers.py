@@ -57,6 +57,8 @@ def random_layer(c, seed=0, x_std=1.0, w_std=0.02, bias_std=0.0):
     if c.dtype == 2:
         from np_restatement import round_bf16
         x, wg, w_up, w_down, b_up, b_down = (round_bf16(a) for a in (x, wg, w_up, w_down, b_up, b_down))
+    if c.dtype == 1:
+        x, wg, w_up, w_down, b_up, b_down = (moe_ref.round_tf32(a) for a in (x, wg, w_up, w_down, b_up, b_down))
     if c.dtype == 3:
         x, wg, w_up, w_down, b_up, b_down = (a.astype(np.float16).astype(np.float32)
                                              for a in (x, wg, w_up, w_down, b_up, b_down))

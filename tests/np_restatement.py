@@ -28,11 +28,22 @@ def round_bf16(a: np.ndarray) -> np.ndarray:
     return (r & 0xFFFFFFFF).astype(np.uint32).view(np.float32).reshape(a.shape)
 
 
+def round_tf32(a: np.ndarray) -> np.ndarray:
+    """fp32 -> tf32 (10 mantissa bits, round to nearest even) -> fp32, by decomposing the value: the
+    mantissa scaled to an integer of 11 bits, rounded by numpy's rint (ties to even), scaled back."""
+    a = np.asarray(a, dtype=np.float32)
+    m, e = np.frexp(a.astype(np.float64))          # a = m * 2^e, 0.5 <= |m| < 1
+    return np.ldexp(np.rint(m * 2048.0) / 2048.0, e).astype(np.float32)
+
+
 def to_elem(a, bf16):
-    """bf16: True / "bf16" -> bfloat16, "f16" -> IEEE half (numpy's conversion), False -> fp32."""
+    """bf16: True / "bf16" -> bfloat16, "f16" -> IEEE half (numpy's conversion), "tf32" -> 10 mantissa
+    bits in 32, False -> fp32."""
     a = np.asarray(a, dtype=np.float32)
     if bf16 == "f16":
         return a.astype(np.float16).astype(np.float32)
+    if bf16 == "tf32":
+        return round_tf32(a)
     return round_bf16(a) if bf16 else a
 
 

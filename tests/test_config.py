@@ -21,14 +21,10 @@ def test_parse_shipped_config_keys():
     cfg = ka.KleosConfig.from_json_text(json.dumps(SHIPPED))
     assert cfg.num_experts == 64 and cfg.expert_top_k == 2 and cfg.sequence_len == 8192
     assert cfg.torch_dtype == 1 and cfg.capacity_factor == 1.0
-    # the shipped dtype is tf32, which CDNA4 does not have: refused by name, not silently changed
-    with pytest.raises(ka.KleosError) as ei:
-        cfg.derive()
-    assert ei.value.code == _capi.KLEOS_EUNSUPPORTED and "tf32" in ei.value.message
-    # the message names the remedy, and the remedy works: the same keys with torch_dtype 2 are the headline layer
-    assert 'set "torch_dtype" to 2' in ei.value.message
-    d = ka.KleosConfig.from_json_text(json.dumps({**SHIPPED, "torch_dtype": 2})).derive()
-    assert (d.S, d.H, d.I, d.E, d.k, d.EC) == (8192, 2048, 2048, 64, 2, 256)
+    # the shipped dtype is tf32: Elements of 32 bits, the derived constants of the headline layer
+    d = cfg.derive()
+    assert (d.S, d.H, d.I, d.E, d.k, d.EC, d.PX, d.elem_bytes) == (8192, 2048, 2048, 64, 2, 256, 64, 4)
+    assert d.in_elems == 8192 * 2048 + 64 * 2048 + 2 * 64 * 2048 * 2048 + 64 * 4096
 
 
 @pytest.mark.parametrize("name,S,PX,EC,pEC,in_elems", [

@@ -356,3 +356,46 @@ def test_layer_fp16_vs_numpy_restatement(oracle):
     np.testing.assert_array_equal(got["topk_expert"], ref["topk_expert"])
     np.testing.assert_array_equal(got["topk_slot"], ref["topk_slot"])
     assert rel_fro(got["moe_out"], ref["moe_out"]) < 2e-3
+
+
+def test_tf32_round_matches_an_independent_rounding(oracle):
+    """tf32 keeps 10 mantissa bits. The oracle rounds on the bit pattern (add, mask); pinned against a
+    rounding that never looks at bits (frexp, rint on the scaled mantissa, ldexp), on random values,
+    exact ties (which go to the even neighbour), a carry into the exponent, and the special values."""
+    lib = oracle.lib()
+    rng = np.random.default_rng(11)
+    vals = np.concatenate([rng.standard_normal(4000).astype(np.float32) * 3.0,
+                           rng.standard_normal(2000).astype(np.float32) * 1e-20,
+                           np.array([1.0 + 2.0 ** -11, 1.0 + 3 * 2.0 ** -11, 1.0 + 2.0 ** -11 + 2.0 ** -20,
+                                     2.0 - 2.0 ** -12, -(2.0 - 2.0 ** -12), 0.0, -0.0, 65504.0, 3.0e38], np.float32)])
+    got = np.array([lib.moe_ref_round_tf32(float(v)) for v in vals], np.float32)
+    np.testing.assert_array_equal(got, npr.round_tf32(vals))
+    np.testing.assert_array_equal(got, oracle.round_tf32(vals))        # the wrapper's numpy form of the same bits
+    assert (got.view(np.uint32) & 0x1FFF == 0).all()
+    assert lib.moe_ref_round_tf32(1.0 + 2.0 ** -11) == 1.0                       # tie: down to the even mantissa
+    assert lib.moe_ref_round_tf32(1.0 + 3 * 2.0 ** -11) == 1.0 + 2.0 ** -9       # tie: up to the even mantissa
+    assert lib.moe_ref_round_tf32(2.0 - 2.0 ** -12) == 2.0                       # carries into the exponent
+    assert np.isinf(lib.moe_ref_round_tf32(float("inf"))) and np.isnan(lib.moe_ref_round_tf32(float("nan")))
+    # what a tensor core reads of an operand: the lower 13 bits dropped, nothing rounded
+    assert lib.moe_ref_tf32_operand(1.0 + 2.0 ** -10 + 2.0 ** -11 + 2.0 ** -12) == 1.0 + 2.0 ** -10
+
+
+def test_layer_tf32_vs_numpy_restatement(oracle):
+    """Whole layer with tf32 Elements against the independent restatement; then the same layer with the
+    lower mantissa bits of x and the weights filled in: a tf32 matrix product does not see them, the
+    bias add does (it reads the stored 32 bits)."""
+    c = oracle.make_cfg(S=128, H=64, I=128, E=8, k=2, dtype=1)
+    x, wg, w_up, w_down, b_up, b_down = random_layer(c, seed=4, w_std=0.1, bias_std=0.05)
+    iP = pack_inputs(c, x, wg, w_up, w_down, b_up, b_down)
+    got = oracle.forward(c, iP)
+    ref = npr.forward(x, wg, w_up, w_down, b_up, b_down, k=2, elem="tf32")
+    np.testing.assert_array_equal(got["topk_expert"], ref["topk_expert"])
+    np.testing.assert_array_equal(got["topk_slot"], ref["topk_slot"])
+    assert rel_fro(got["moe_out"], ref["moe_out"]) < 2e-3
+    assert (got["moe_out"].view(np.uint32) & 0x1FFF == 0).all() and (got["gate_out"].view(np.uint32) & 0x1FFF == 0).all()
+    noisy = iP.copy()
+    n_mm = c.S * c.H + c.PX * c.H + 2 * c.E * c.I * c.H          # everything in front of the bias vectors
+    noisy[:n_mm] = (noisy[:n_mm].view(np.uint32) | 0x0ABC).view(np.float32)
+    again = oracle.forward(c, noisy)
+    np.testing.assert_array_equal(again["moe_out"], got["moe_out"])
+    np.testing.assert_array_equal(again["logits"], got["logits"])
