@@ -167,15 +167,18 @@ __device__ __forceinline__ void static_for(F&& f) {
 // AHEAD2 (two stages only): the loads run two slices ahead, at the price of a second workgroup
 // barrier per slice. It pays where the weights stream from HBM and a slice's loads take longer than
 // its matrix work (headline shape: 301 against 315 us for the expert phase); where the matrix work
-// dominates the extra barrier costs more than the earlier loads bring (8-expert shape with hidden
-// size 4096: 4.22 against 4.03 ms).
+// dominates it needs SPREAD to pay (8-expert shape with hidden size 4096, both projections: 4.18 ms
+// with all loads of a slice at once against 4.11 one slice ahead, 3.95 with them shared out 4 + 4).
 // SPREAD (with AHEAD2): when the loads of a slice are issued. 0: all of them behind the matrix
 // instructions of the last K step of the slice two before it, which frees their stage. Otherwise
-// only the first of them go there and the rest behind the first three K steps of the next slice
-// (spread_count): the CU's load path takes in one 1 KB load about every 36 clocks while all CUs
-// stream, so the 64 loads of a slice issued by eight wavefronts inside one K step hold every
-// wavefront - and with it its matrix instructions, which sit behind the loads in program order -
-// for as long as four K steps of matrix work take.
+// only the first of them go there and the rest behind the first K steps of the next slice
+// (spread_count: 1 = 4 + 4, 2 = 3 + 3 + 2 of the 8 loads of a wavefront). The CU's load path takes in
+// about one 1 KB load every 36 clocks while all CUs stream; the 64 loads of a slice issued by eight
+// wavefronts inside one K step queue up in front of it, and each wavefront's matrix instructions sit
+// behind its loads in program order. Shared out evenly over all four K steps the last loads leave too
+// late (4.07 ms at the shape above); one barrier per slice instead of two (the barrier in front of the
+// last K step also standing for "the next slice has landed", its first fragments read behind that K
+// step's matrix instructions) loses the lead time it needs: 3.98 ms.
 template <typename E, int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES, bool STREAM_B, bool AHEAD2, int SPREAD = 0>
 struct Gemm16 {
     typedef typename Elem16<E>::vec8 vec8;

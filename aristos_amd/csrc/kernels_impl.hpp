@@ -36,7 +36,7 @@ constexpr int kXcds = 8;
 // Expert GEMM configuration of the bf16 / fp16 path: 256 x 256 tile (an expert's whole capacity of
 // 256 rows at the headline shape, so its weights stream from HBM exactly once), 4 x 2 wavefronts of
 // 64 x 128 (two per SIMD), K slices of 64 (whole 128-byte lines of every row) through two 64 KB
-// stages, loads two slices ahead.
+// stages, loads two slices ahead, a slice's loads shared out 3 + 3 + 2 over three K steps.
 // (Measured against it on MI355X, none faster: K slices of 32 through four stages, 2 x 2 wavefronts
 // of 128 x 128 with the accumulators in AGPRs, weight slices of 64 through three slots with
 // activation half slices of 32 through three, the 128 x 256 tile of variant 1. 2 x 4 wavefronts
@@ -49,7 +49,9 @@ constexpr int kXcds = 8;
 // Variant 2, for layers whose experts hold at least four row blocks (few large experts: every
 // weight tile is shared by several workgroups through L2, loads return quickly and the matrix work
 // dominates): the tile of variant 0 on 2 x 4 wavefronts of 128 x 64 (3.53 against 3.57 ms with 4 x 2
-// at the 8-expert shape with hidden size 4096), the loads one slice ahead, issued during the first K step.
+// at the 8-expert shape with hidden size 4096), the loads two slices ahead like variant 0 and shared
+// out 4 + 4 over two K steps (both projections of that shape on random data: 3.95 ms against 4.11 with
+// the loads one slice ahead, all behind the first K step, and 4.18 two slices ahead all at once).
 // Variants 0 and 1 load their weight rows non-temporally (headline 378 against 390 us per forward,
 // the 16-expert shape 192 against 196, the 256-expert shape 3.43 against 3.48 ms); variant 2, whose
 // weight tiles are shared by eight workgroups and more, does not (4.06 against 4.01 ms with it).
@@ -75,6 +77,7 @@ using GemmCfg = std::conditional_t<V == 0, Gemm16<E, 256, 256, 4, 2, 64, 2, true
 // matrix instruction, so which tile computed a row does not show in its bits.)
 template <typename E, int V>
 using NarrowCfg = Gemm16<E, 128, 256, 2, 4, 64, 3, false, false>;
+template <typename G> struct TypeTag { using type = G; };   // a type handed to a generic lambda
 template <typename T, int V> constexpr bool kMixedHeights = sizeof(T) == 2 && V == 2 && KLEOS_TUNE_MIXED_HEIGHTS != 0;
 constexpr uint32_t kNarrowTileRows = 128;
 constexpr int kBN = 256;
@@ -447,15 +450,13 @@ __device__ __forceinline__ void expert_loop(const LayerParams& p, char* smem, ui
                 G::begin(cur_t, args_of(cur), G::next_stage0(cur_t), bias_slot ^= 1, smem);
             }
         };
-        struct WideTag { using type = GemmCfg<T, V>; };
-        struct NarrowTag { using type = NarrowCfg<T, V>; };
         Task t = next();
         while (t.valid) {
             if constexpr (kMixedHeights<T, V>) {
-                if (t.narrow) t = run(NarrowTag{}, std::true_type{}, t);
-                else t = run(WideTag{}, std::false_type{}, t);
+                if (t.narrow) t = run(TypeTag<NarrowCfg<T, V>>{}, std::true_type{}, t);
+                else t = run(TypeTag<GemmCfg<T, V>>{}, std::false_type{}, t);
             } else {
-                t = run(WideTag{}, std::false_type{}, t);
+                t = run(TypeTag<GemmCfg<T, V>>{}, std::false_type{}, t);
             }
         }
         flush_stats();
@@ -929,7 +930,7 @@ size_t fused_smem_bytes(uint32_t E) {
     return need;
 }
 
-int gate_groups(uint32_t E) {
+inline int gate_groups(uint32_t E) {
     const uint32_t g = ceil_div_u32(E, 16);
     if (g <= 1) return 1;
     if (g <= 2) return 2;
