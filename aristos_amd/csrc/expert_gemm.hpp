@@ -59,6 +59,7 @@ struct GemmTileArgs {
     const elem16_t* a_base;        // A rows (gathered through a_row_index when it is not null)
     const int32_t* a_row_index;
     uint32_t a_rows;               // rows behind a_base: gathered indices are clamped below it
+    const elem16_t* a_pad;         // K zeros that stand in for the rows past m_valid (null: they re-read the last valid row)
     const elem16_t* b_base;        // first of the tile's weight rows
     const elem16_t* bias;          // first of the tile's bias entries
     elem16_t* c_base;              // output element (row 0, column 0) of the tile
@@ -283,8 +284,10 @@ struct Gemm16 {
     }
 
     // Per-lane source addresses, the load of the bias into LDS slot `bias_slot`, then the loads of
-    // the first STAGES-1 slices. Rows past the valid range re-read the last valid row: their
-    // products land in accumulator rows / columns that are never stored. The stages stage0 ..
+    // the first STAGES-1 slices. Activation rows past the valid range read zeros (a_pad; the last valid
+    // row without it) and weight rows past it re-read the last valid row: their products land in
+    // accumulator rows / columns that are never stored, and a matrix core that multiplies zeros draws
+    // less power than one that multiplies data. The stages stage0 ..
     // stage0+STAGES-2 and the bias slot must not be in use by any wavefront. The bias load is the
     // oldest of the tile's loads, so the first wait of mainloop() covers it.
     static __device__ __forceinline__ void begin(Tile& t, const GemmTileArgs& g, int stage0, int bias_slot, char* smem) {
@@ -314,7 +317,9 @@ struct Gemm16 {
 #pragma unroll
         for (int i = 0; i < LA; ++i) {
             const int row = kRowsPerLoad * (wave + kWaves * i) + ld_r;
-            t.pa[i] = g.a_base + size_t(src[i]) * g.lda + ((ld_p ^ swizzle(row)) << 3);
+            const elem16_t* from = g.a_base + size_t(src[i]) * g.lda;
+            if (g.a_pad && row >= int(g.m_valid)) from = g.a_pad;
+            t.pa[i] = from + ((ld_p ^ swizzle(row)) << 3);
         }
 #pragma unroll
         for (int i = 0; i < LB; ++i) {

@@ -62,6 +62,12 @@ constexpr int kXcds = 8;
 #ifndef KLEOS_TUNE_V2_SPREAD
 #define KLEOS_TUNE_V2_SPREAD 1       // variant 2: two slices ahead, 4 + 4 over two K steps; -1: one slice ahead
 #endif
+#ifndef KLEOS_TUNE_ZERO_PAD
+#define KLEOS_TUNE_ZERO_PAD 1      // activation rows past an expert's last row read zeros instead of its last row
+#endif
+#ifndef KLEOS_TUNE_HALVED_TAIL
+#define KLEOS_TUNE_HALVED_TAIL 1   // dynamic schedule: the last down-projection tiles of a queue as halves of 128 rows
+#endif
 #ifndef KLEOS_TUNE_MIXED_HEIGHTS
 #define KLEOS_TUNE_MIXED_HEIGHTS 1   // variant 2: 128-row tiles for last row blocks of at most 128 rows
 #endif
@@ -80,6 +86,9 @@ using NarrowCfg = Gemm16<E, 128, 256, 2, 4, 64, 3, false, false>;
 template <typename G> struct TypeTag { using type = G; };   // a type handed to a generic lambda
 template <typename T, int V> constexpr bool kMixedHeights = sizeof(T) == 2 && V == 2 && KLEOS_TUNE_MIXED_HEIGHTS != 0;
 constexpr uint32_t kNarrowTileRows = 128;
+// What the padding rows of an expert tile read: zeros, as long as the inner dimension is no longer than this.
+constexpr int kZeroRowElems = 16384;
+static __device__ __attribute__((aligned(256))) const elem16_t g_zero_row[kZeroRowElems] = {};
 constexpr int kBN = 256;
 constexpr int kGemmThreads = GemmCfg<bf16_t, 0>::kThreads;
 static_assert(NarrowCfg<bf16_t, 2>::kThreads == kGemmThreads, "both tile heights run on the same workgroup");
@@ -253,7 +262,8 @@ struct Task {
     uint32_t foreign;   // taken from another XCD's queue: its h1 rows may sit in a different L2
     uint32_t dep;       // down tile: the readiness counter of its row block as seen when handed out
     uint32_t ready;     // down tile whose up-projection row block was already complete when handed out
-    uint32_t narrow;    // the row block holds at most 128 rows and goes to the 128-row tile (layers that mix tile heights)
+    uint32_t narrow;    // goes to the 128-row tile (layers that mix tile heights): a row block of at most 128 rows, or one half of a row block
+    uint32_t half;      // narrow tile that starts 128 rows into its row block (the second half of a halved block)
     uint32_t valid;
 };
 constexpr int kTaskWords = 12;
@@ -264,13 +274,13 @@ __device__ __forceinline__ Task broadcast_task(uint32_t* s_task, const Task& min
     if (threadIdx.x == 0) {
         s_task[0] = mine.e; s_task[1] = mine.kind; s_task[2] = mine.mtile; s_task[3] = mine.ntile;
         s_task[4] = mine.foreign; s_task[5] = mine.ready; s_task[6] = mine.valid; s_task[7] = mine.rows;
-        s_task[8] = mine.dep; s_task[9] = mine.narrow;
+        s_task[8] = mine.dep; s_task[9] = mine.narrow; s_task[10] = mine.half;
     }
     __syncthreads();
     Task t;
     t.e = s_task[0]; t.kind = s_task[1]; t.mtile = s_task[2]; t.ntile = s_task[3];
     t.foreign = s_task[4]; t.ready = s_task[5]; t.valid = s_task[6]; t.rows = s_task[7];
-    t.dep = s_task[8]; t.narrow = s_task[9];
+    t.dep = s_task[8]; t.narrow = s_task[9]; t.half = s_task[10];
     return t;
 }
 
@@ -285,10 +295,11 @@ __device__ __forceinline__ TileOperands<T> tile_operands(const LayerParams& p, c
     constexpr int BM = TileShape<T, V>::BM, BN = TileShape<T, V>::BN;
     TileOperands<T> o;
     const uint32_t rows = t.rows;
-    const uint32_t row0 = t.mtile * BM, col0 = t.ntile * BN;
+    const uint32_t row0 = t.mtile * BM + t.half * kNarrowTileRows, col0 = t.ntile * BN;
     const uint32_t N = t.kind == 0 ? p.I : p.H;
+    const uint32_t height = t.narrow ? kNarrowTileRows : uint32_t(BM);
     o.K = t.kind == 0 ? p.H : p.I;
-    o.m_valid = rows - row0 < uint32_t(BM) ? rows - row0 : uint32_t(BM);
+    o.m_valid = rows - row0 < height ? rows - row0 : height;
     o.n_valid = N - col0 < uint32_t(BN) ? N - col0 : uint32_t(BN);
     o.w = static_cast<const T*>(t.kind == 0 ? p.w_up : p.w_down) + size_t(t.e) * p.I * p.H + size_t(col0) * o.K;
     o.bias = static_cast<const T*>(t.kind == 0 ? p.b_up : p.b_down) + size_t(t.e) * N + col0;
@@ -397,6 +408,7 @@ __device__ __forceinline__ void expert_loop(const LayerParams& p, char* smem, ui
             const TileOperands<T> o = tile_operands<T, V>(p, t);
             GemmTileArgs g;
             g.a_base = reinterpret_cast<const elem16_t*>(o.a); g.a_row_index = o.idx; g.a_rows = p.S;
+            g.a_pad = KLEOS_TUNE_ZERO_PAD != 0 && o.K <= uint32_t(kZeroRowElems) ? g_zero_row : nullptr;
             g.b_base = reinterpret_cast<const elem16_t*>(o.w); g.bias = reinterpret_cast<const elem16_t*>(o.bias);
             g.c_base = reinterpret_cast<elem16_t*>(o.c);
             g.lda = o.lda; g.ldb = o.K; g.ldc = o.ldc; g.K = o.K; g.m_valid = o.m_valid; g.n_valid = o.n_valid;
@@ -506,7 +518,7 @@ __device__ __forceinline__ void gate_gemm_phase(const LayerParams& p, char* smem
         const uint32_t k0 = (slices * split) / splits, k1 = (slices * (split + 1)) / splits;
         GemmTileArgs g;
         g.a_base = static_cast<const elem16_t*>(p.x) + size_t(mb) * kGateTileM * p.H + size_t(k0) * G::kSliceK;
-        g.a_row_index = nullptr; g.a_rows = p.S;
+        g.a_row_index = nullptr; g.a_rows = p.S; g.a_pad = nullptr;
         g.b_base = static_cast<const elem16_t*>(p.wg) + size_t(nb) * kGateTileN * p.H + size_t(k0) * G::kSliceK;
         g.bias = static_cast<const elem16_t*>(p.wg);   // any readable 512 bytes: the sums take no bias
         g.c_base = nullptr;
@@ -691,7 +703,10 @@ __global__ __launch_bounds__((TileShape<T, V>::kThreads), (TileShape<T, V>::kPer
     // workgroup, [5] every XCD holds the same number of workgroups. Thread 0's own words live here
     // rather than in registers that would stay occupied through the GEMM main loop.
     uint32_t* s_static = s_qup + 8;
-    static_assert((16 + 8 + kTaskWords + 8 + 6) * 4 <= kLdsQueue, "queue header");
+    // [8] the ticket from which a queue hands out its last down-projection tiles as halves of 128
+    // rows, two tickets per tile (~0: none)
+    uint32_t* s_qhalf = s_static + 6;
+    static_assert((16 + 8 + kTaskWords + 8 + 6 + 8) * 4 <= kLdsQueue, "queue header");
     Segment* s_seg = reinterpret_cast<Segment*>(smem + lds_queue_offset(p.E) + kLdsQueue);   // at most 2*E segments
     char* s_gemm = smem + fused_lds_header(p.E);
     const uint32_t tn_up = ceil_div_u32(p.I, BN), tn_down = ceil_div_u32(p.H, BN);
@@ -839,7 +854,21 @@ __global__ __launch_bounds__((TileShape<T, V>::kThreads), (TileShape<T, V>::kPer
                     ticket += uint32_t(s_mt[e]) * tn_down;
                 }
             }
-            s_qtot[q] = ticket;
+            // Freely handed-out tiles end raggedly: the workgroups of an XCD run in step, so a last
+            // round that is not full leaves the others idle for a whole tile, and a workgroup of
+            // another XCD that takes one of the last tiles finishes a whole tile later. Where the
+            // kernel holds both tile heights, the last down-projection tiles of a queue (half a round's
+            // worth) are therefore handed out as two tickets of 128 rows each. What a tile computes
+            // does not depend on its height (same instructions, same order along K).
+            uint32_t halved = 0;
+            if constexpr (kMixedHeights<T, V> && KLEOS_TUNE_HALVED_TAIL != 0) {
+                if (!use_static && nq != 0 && lag != 0) {
+                    const uint32_t last = uint32_t(s_mt[expert_at(q, nq - 1)]) * tn_down;   // the queue ends with this expert's down tiles
+                    halved = last < members / 2 ? last : members / 2;
+                }
+            }
+            s_qhalf[q] = halved ? ticket - halved : ~0u;
+            s_qtot[q] = ticket + halved;
             s_qup[q] = ups;
         }
         __syncthreads();
@@ -850,7 +879,16 @@ __global__ __launch_bounds__((TileShape<T, V>::kThreads), (TileShape<T, V>::kPer
     uint32_t q_dead = 0;  // bit q: queue q was seen exhausted
     bool q_scanned = false;
     const Readiness rd{sched, mt_max, tn_up, p.wait_ticks};
-    auto decode = [&](Task& t, uint32_t q, uint32_t ticket) {
+    // Fills in the tile behind a ticket; false for a ticket that stands for no rows (the second
+    // half of a halved row block that holds at most 128 rows).
+    auto decode = [&](Task& t, uint32_t q, uint32_t ticket) -> bool {
+        uint32_t half = 0, halved = 0;
+        const uint32_t from = s_qhalf[q];
+        if (ticket >= from) {   // two tickets per tile from here on
+            half = (ticket - from) & 1u;
+            halved = 1;
+            ticket = from + (ticket - from) / 2;
+        }
         uint32_t sg = s_qseg[q];
         const uint32_t sg_end = s_qseg[q + 1];
         while (sg + 1 < sg_end && s_seg[sg + 1].start <= ticket) ++sg;
@@ -861,14 +899,18 @@ __global__ __launch_bounds__((TileShape<T, V>::kThreads), (TileShape<T, V>::kPer
         t.ntile = local / s_mt[t.e];
         t.rows = s_rows[t.e];
         t.narrow = narrow_block<T, V>(t.rows, t.mtile);
+        if (half && t.narrow) return false;   // the first half held all its rows
+        t.narrow |= halved;
+        t.half = half;
         t.valid = 1;
+        return true;
     };
     auto next = [&]() {
         Task t{};
         if (tid == 0 && use_static) {
             const uint32_t ticket = s_static[3];
             if (ticket < s_qtot[xcd]) {
-                decode(t, xcd, ticket);
+                decode(t, xcd, ticket);   // (no halved tiles in the static schedule)
                 t.dep = t.kind == 0 ? 0u : atomic_load_relaxed(rd.counter(t));
                 t.ready = t.kind == 0 || rd.complete(t.dep);
                 s_static[3] = ticket + members;
@@ -888,7 +930,7 @@ __global__ __launch_bounds__((TileShape<T, V>::kThreads), (TileShape<T, V>::kPer
                 if (s_qtot[q] == 0 || ((q_dead >> q) & 1u)) { ++q_off; continue; }
                 const uint32_t ticket = atomic_add_agent(sched + kSchedTicket + q * kSchedLine, 1u);
                 if (ticket >= s_qtot[q]) { ++q_off; continue; }
-                decode(t, q, ticket);
+                if (!decode(t, q, ticket)) continue;
                 t.foreign = q_off != 0;
                 t.dep = t.kind == 0 ? 0u : atomic_load_relaxed(rd.counter(t));
                 t.ready = t.kind == 0 || rd.complete(t.dep);

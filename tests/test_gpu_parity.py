@@ -301,6 +301,57 @@ def test_tile_heights_mixed_inside_one_layer(mode, k):
     assert (v["topk_slot"] >= 0).all()
 
 
+def test_last_down_tiles_of_a_queue_are_handed_out_in_halves():
+    """Dynamic schedule of a layer that holds both tile heights: every XCD queue hands out its last
+    down-projection tiles (as many as half of the XCD's workgroups) as two tickets of 128 rows each,
+    except where a last block holds at most 128 rows anyway. The persistent launch therefore counts
+    more tiles than row blocks x column tiles, by a number the test works out from the rows per expert,
+    and its output has the bits of the separate launches per phase, which never halve a tile."""
+    S, H, I, E, k = 3072, 512, 256, 8, 2
+    keys = _keys(S, H, I, E, k, cf=1.0, drop=0)
+    c = moe_ref.cfg_from_keys(keys)
+    assert c.cap_rows >= 1024
+    x, wg, w_up, w_down, b_up, b_down = random_layer(c, seed=93, w_std=0.08, bias_std=0.1)
+    rows = [40, 100, 129, 300, 2100, 403, 0, 0]
+    first = np.repeat(np.arange(E), rows)
+    np.random.default_rng(6).shuffle(first)
+    x[:, :E] = 0.0
+    x[np.arange(S), first] = 8.0
+    x[np.arange(S), (first + 1) % E] = 4.0
+    wg[:, :E] = np.eye(E, dtype=np.float32)
+    wg[:, E:] *= 0.25
+    iP_np = pack_inputs(c, x, wg, w_up, w_down, b_up, b_down)
+    iP = _to_device(c, iP_np)
+    _, ref, v = run_gpu(keys, iP, ka.MODE_PHASED)
+    ref = _out_to_np(c, ref)
+    kept = np.array(rows) + np.roll(rows, 1)
+    np.testing.assert_array_equal(v["expert_count"], kept)
+    d = ka.initialize(keys)
+    try:
+        ka.moe.set_mode(ka.MODE_FUSED)
+        ka.moe.set_schedule(ka.SCHEDULE_DYNAMIC)
+        oP = synth.alloc_outputs(d)
+        ka.moe.forward_host(iP, oP)
+        ka.moe.stream_synchronize()
+        np.testing.assert_array_equal(_out_to_np(c, oP), ref)
+        ka.moe.forward_host_bench(iP, oP, skip=1, trials=2)
+        np.testing.assert_array_equal(_out_to_np(c, oP), ref)
+        st = ka.moe.scheduler_stats()
+        members = ka.moe.phase_stamps().shape[0] // 8        # workgroups per XCD
+    finally:
+        ka.finalize()
+    tn_up, tn_down = -(-I // 256), -(-H // 256)
+    expect = 0
+    for r in kept:                                       # by-index placement: queue q holds expert q alone
+        mt = -(-int(r) // 256)
+        expect += mt * (tn_up + tn_down)
+        tiles = [(n, m) for n in range(tn_down) for m in range(mt)]      # row blocks fastest
+        for n, m in tiles[len(tiles) - min(len(tiles), members // 2):]:
+            expect += int(r - m * 256 > 128)             # a second ticket unless the block fits one 128-row tile
+    assert members >= 2 and int(st["tiles"]) == expect
+    assert expect > sum(-(-int(r) // 256) for r in kept) * (tn_up + tn_down)
+
+
 @pytest.mark.parametrize("dt", [2, 0])
 def test_dense_packing_of_a_single_expert(dt):
     """num_experts == 1 on the packing the reference's fffn kernel reads (fffn.cuh:43-49): iP = x | Wup |
