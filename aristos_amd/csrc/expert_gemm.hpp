@@ -50,6 +50,39 @@ namespace kleos_amd {
 typedef const __attribute__((address_space(1))) void* global_cptr;
 typedef __attribute__((address_space(3))) void* lds_ptr;
 
+// One direct global->LDS load: every lane names 16 bytes of global memory, and the 64 lanes' bytes
+// land in the 1 KB of LDS at `dst` (the same address in all lanes; the instruction takes it from M0)
+// in lane order. Written as inline assembly, not as the compiler's builtin, on purpose: the compiler
+// cannot see the `s_waitcnt vmcnt` this file places by hand, so it takes every direct load it knows
+// of for pending for ever, and in front of any later LDS read whose address it cannot tell apart
+// from the loads' destinations it waits for all of them (`vmcnt(0)`) - which empties the pipeline of
+// loads that run one or two K slices ahead. Whether it could tell them apart turned out to depend on
+// the surrounding code (the same main loop lost 11 % inside one kernel and nothing inside another).
+// The ordering these loads need is all explicit here: a wait for the wavefront's own loads, then a
+// workgroup barrier, before anybody reads a stage; a barrier behind everybody's last read before a
+// stage is written again. Loads the compiler does not know of only make its own waits stricter.
+// (M0 is a register the compiler sets up itself right in front of each instruction that reads it
+// and keeps nothing in; it warns about any statement that names it)
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Winline-asm"
+// `lds`: the LDS address of the 1 KB, a value the compiler holds in a scalar register (lds_address()
+// plus offsets that are the same in all lanes).
+template <bool NON_TEMPORAL>
+__device__ __forceinline__ void direct_load16(const void* src, uint32_t lds) {
+    // (one wait state between the write of M0 and the load that reads it)
+    if constexpr (NON_TEMPORAL)
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off nt" ::"s"(lds), "v"(src) : "memory", "m0");
+    else
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds), "v"(src) : "memory", "m0");
+}
+#pragma clang diagnostic pop
+// The LDS address of a pointer into the workgroup's LDS, in a scalar register.
+__device__ __forceinline__ uint32_t lds_address(const char* p) {
+    return __builtin_amdgcn_readfirstlane(uint32_t(reinterpret_cast<uintptr_t>((__attribute__((address_space(3))) const char*)p)));
+}
+// The wavefront's index within the workgroup, in a scalar register.
+__device__ __forceinline__ uint32_t wave_index() { return __builtin_amdgcn_readfirstlane(threadIdx.x >> 6); }
+
 // A 16-bit Element seen only as storage: addresses are computed in units of it, values are
 // interpreted by the Element type the tile is instantiated with.
 typedef uint16_t elem16_t;
@@ -153,6 +186,62 @@ __device__ __forceinline__ void epilogue16(const TileOut& t, f32x16 (&acc)[WN / 
     else epilogue16_act<E, WM, WN, WAVES_N, 2>(t, acc, stage_mem, bias_mem);
 }
 
+// The same epilogue for accumulators of 16 x 16 matrix-core tiles: acc[ni][mi][v] is output column
+// n = wn*WN + ni*16 + 4*(lane/16) + v of output row m = wm*WM + mi*16 + lane%16 - again 4 consecutive
+// columns per lane and tile, so the panels, their LDS layout and the stores are the ones above.
+template <typename E, int WM, int WN, int WAVES_N, int ACT>
+__device__ __forceinline__ void epilogue16_act(const TileOut& t, f32x4 (&acc)[WN / 16][WM / 16], char* stage_mem,
+                                               const char* bias_mem) {
+    typedef typename Elem16<E>::vec4 vec4;
+    constexpr int kPanelRows = kEpiloguePanelRows;
+    const uint32_t tid = local_tid();
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+    const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+    const int fr_row = lane & 15, fr_part = lane >> 4;
+    char* stg = stage_mem + wave * (kPanelRows * 128);
+    const char* bias_lane = bias_mem + (wn * WN + 4 * fr_part) * 2;
+#pragma unroll
+    for (int pm = 0; pm < WM / 32; ++pm) {
+#pragma unroll
+        for (int pn = 0; pn < WN / 64; ++pn) {
+#pragma unroll
+            for (int ml = 0; ml < 2; ++ml) {
+                const int r = ml * 16 + fr_row;   // row of the panel
+#pragma unroll
+                for (int nl = 0; nl < 4; ++nl) {
+                    const int ni = pn * 4 + nl;
+                    const vec4 b4 = *reinterpret_cast<const vec4*>(bias_lane + ni * 16 * 2);
+                    vec4 o;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        o[j] = static_cast<E>(activate<ACT>(acc[ni][pm * 2 + ml][j] + float(b4[j])));
+                    // columns nl*16 + 4*fr_part .. + 3 of the panel: chunk 2*nl + fr_part/2, half fr_part%2
+                    *reinterpret_cast<vec4*>(stg + r * 128 + (((2 * nl + (fr_part >> 1)) ^ ((r >> 1) & 7)) << 4) + (fr_part & 1) * 8) = o;
+                }
+            }
+#pragma unroll
+            for (int it = 0; it < kPanelRows * 8 / kWave; ++it) {
+                const int id = it * kWave + lane;
+                const int r = id >> 3, c = id & 7;
+                const u32x4 v = load16(stg + r * 128 + ((c ^ ((r >> 1) & 7)) << 4));
+                const uint32_t m = wm * WM + pm * 32 + r, n = wn * WN + pn * 64 + c * 8;
+                if (m < t.m_valid && n < t.n_valid) {
+                    constexpr int kAgentScope = 16;   // sc1
+                    __builtin_amdgcn_raw_buffer_store_b128(v, coherent_rows(t.c_base), int((size_t(m) * t.ldc + n) * sizeof(E)), 0,
+                                                           kAgentScope);
+                }
+            }
+        }
+    }
+}
+template <typename E, int WM, int WN, int WAVES_N>
+__device__ __forceinline__ void epilogue16(const TileOut& t, f32x4 (&acc)[WN / 16][WM / 16], char* stage_mem,
+                                           const char* bias_mem) {
+    if (t.act == 0) epilogue16_act<E, WM, WN, WAVES_N, 0>(t, acc, stage_mem, bias_mem);
+    else if (t.act == 1) epilogue16_act<E, WM, WN, WAVES_N, 1>(t, acc, stage_mem, bias_mem);
+    else epilogue16_act<E, WM, WN, WAVES_N, 2>(t, acc, stage_mem, bias_mem);
+}
+
 // f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>), in this order.
 template <int N, typename F>
 __device__ __forceinline__ void static_for(F&& f) {
@@ -180,14 +269,20 @@ __device__ __forceinline__ void static_for(F&& f) {
 // late (4.07 ms at the shape above); one barrier per slice instead of two (the barrier in front of the
 // last K step also standing for "the next slice has landed", its first fragments read behind that K
 // step's matrix instructions) loses the lead time it needs: 3.98 ms.
-template <typename E, int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES, bool STREAM_B, bool AHEAD2, int SPREAD = 0>
+// MI: the matrix-core tile. 32: 32x32x16 instructions (16 values of K each, 16 accumulator registers);
+// 16: 16x16x32 instructions (32 values of K, 4 accumulator registers). The smaller tile reads and
+// writes half as many accumulator registers per multiply-add and draws less power for the same work
+// (instruction loops on random bf16 operands held in registers, whole device: 2.08 against 1.84
+// PFLOP/s at the same 1.31 kW), which is what bounds these kernels.
+template <typename E, int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES, bool STREAM_B, bool AHEAD2, int SPREAD = 0, int MI = 32>
 struct Gemm16 {
     typedef typename Elem16<E>::vec8 vec8;
     typedef typename Elem16<E>::vec4 vec4;
     static constexpr int kWaves = WAVES_M * WAVES_N;
     static constexpr int kThreads = kWaves * kWave;
     static constexpr int WM = BM / WAVES_M, WN = BN / WAVES_N;     // wavefront tile
-    static constexpr int TM = WM / 32, TN = WN / 32;               // 32x32 matrix-core tiles per wavefront
+    static constexpr int TM = WM / MI, TN = WN / MI;               // matrix-core tiles per wavefront
+    static constexpr int KI = MI == 32 ? 16 : 32;                  // values of K one matrix instruction consumes
     static constexpr int kRowBytes = BK * 2;
     static constexpr int kRowsPerLoad = 1024 / kRowBytes;          // rows one direct load covers
     static constexpr int kChunks = kRowBytes / 16;                 // 16-byte chunks per row
@@ -198,9 +293,10 @@ struct Gemm16 {
     static constexpr int kSmemBytes = STAGES * kStage + 2 * kBiasBytes;
     static constexpr int LA = BM / (kRowsPerLoad * kWaves), LB = BN / (kRowsPerLoad * kWaves);
     static constexpr int kLoadsPerSlice = LA + LB;                 // per wavefront
-    static constexpr int kNonTemporal = 2;                         // cache policy bit nt of a load
     static constexpr int kSliceK = BK;                             // values of K per slice
-    static constexpr int kSteps = BK / 16;                         // matrix instructions consume 16 values of K
+    static constexpr int kSteps = BK / KI;                         // K steps per slice
+    static constexpr int kQuarters = 4;                            // a slice's matrix instructions in four equal runs
+    static constexpr int kPerQuarter = TN * TM * kSteps / kQuarters;
     static constexpr int kPanelRows = kEpiloguePanelRows;          // epilogue staging: 32 rows x 64 columns per wavefront
     // loads of a slice (per wavefront) issued at the last K step of the slice two before it [0] and at
     // K steps 0, 1, 2 of the slice before it [1..3]
@@ -216,6 +312,8 @@ struct Gemm16 {
     static_assert(SPREAD == 0 || (AHEAD2 && (LA + LB) % 8 == 0));
     static_assert(spread_count(0) + spread_count(1) + spread_count(2) + spread_count(3) == LA + LB);
     static_assert(BK == 32 || BK == 64);
+    static_assert(MI == 32 || MI == 16);
+    static_assert(kQuarters % kSteps == 0 && (TN * TM * kSteps) % kQuarters == 0);
     static_assert(!AHEAD2 || STAGES == 2);
     static_assert(STAGES >= 2 && STAGES <= 4);
     static_assert(WM % 32 == 0 && WN % 64 == 0);
@@ -239,43 +337,41 @@ struct Gemm16 {
         int bias_slot;              // which of the two LDS bias slots holds this tile's bias
     };
 
-    typedef f32x16 Acc[TN][TM];
+    typedef std::conditional_t<MI == 32, f32x16, f32x4> AccTile;
+    typedef AccTile Acc[TN][TM];
 
     static __device__ __forceinline__ int stage_of(const Tile& t, uint32_t kt) { return (t.stage0 + kt) % STAGES; }
 
     // the direct loads that bring K slice kt of the tile into its stage: activation rows first (they
     // come from L2 and return early), then the weight rows
     static __device__ __forceinline__ void issue_slice(const Tile& t, char* smem, uint32_t kt) {
-        const int wave = threadIdx.x >> 6;
-        char* sa = smem + stage_of(t, kt) * kStage;
-        char* sb = sa + kABytes;
+        const uint32_t sa = lds_address(smem) + stage_of(t, kt) * kStage + 1024 * wave_index();   // this wavefront's first KB of the stage
+        const uint32_t sb = sa + kABytes;
         uint32_t slice = kt + t.k_first;
         slice = slice >= t.k_tiles ? slice - t.k_tiles : slice;
         const uint32_t k0 = slice * BK;
 #pragma unroll
         for (int i = 0; i < LA; ++i)
-            __builtin_amdgcn_global_load_lds((global_cptr)(t.pa[i] + k0), (lds_ptr)(sa + 1024 * (wave + kWaves * i)), 16, 0, 0);
+            direct_load16<false>(t.pa[i] + k0, sa + 1024 * kWaves * i);
 #pragma unroll
         for (int i = 0; i < LB; ++i)
-            __builtin_amdgcn_global_load_lds((global_cptr)(t.pb[i] + k0), (lds_ptr)(sb + 1024 * (wave + kWaves * i)), 16, 0,
-                                             STREAM_B ? kNonTemporal : 0);
+            direct_load16<STREAM_B>(t.pb[i] + k0, sb + 1024 * kWaves * i);
     }
 
     // Load number j (0 <= j < LA + LB) of a K slice: activation rows first (they come from L2 and return
     // early), then the weight rows.
-    static __device__ __forceinline__ void issue_one(const Tile& t, char* sa, char* sb, uint32_t k0, int j) {
-        const int wave = threadIdx.x >> 6;
+    // (sa, sb: the LDS addresses of this wavefront's first KB of the stage's activation and weight rows)
+    static __device__ __forceinline__ void issue_one(const Tile& t, uint32_t sa, uint32_t sb, uint32_t k0, int j) {
         if (j >= LA)
-            __builtin_amdgcn_global_load_lds((global_cptr)(t.pb[j - LA] + k0), (lds_ptr)(sb + 1024 * (wave + kWaves * (j - LA))), 16, 0,
-                                             STREAM_B ? kNonTemporal : 0);
+            direct_load16<STREAM_B>(t.pb[j - LA] + k0, sb + 1024 * kWaves * (j - LA));
         else
-            __builtin_amdgcn_global_load_lds((global_cptr)(t.pa[j] + k0), (lds_ptr)(sa + 1024 * (wave + kWaves * j)), 16, 0, 0);
+            direct_load16<false>(t.pa[j] + k0, sa + 1024 * kWaves * j);
     }
     // Loads first .. first + count - 1 of K slice kt.
     template <int FIRST, int COUNT>
     static __device__ __forceinline__ void issue_range(const Tile& t, char* smem, uint32_t kt) {
-        char* sa = smem + stage_of(t, kt) * kStage;
-        char* sb = sa + kABytes;
+        const uint32_t sa = lds_address(smem) + stage_of(t, kt) * kStage + 1024 * wave_index();
+        const uint32_t sb = sa + kABytes;
         uint32_t slice = kt + t.k_first;
         slice = slice >= t.k_tiles ? slice - t.k_tiles : slice;
         const uint32_t k0 = slice * BK;
@@ -296,7 +392,7 @@ struct Gemm16 {
         const int ld_r = lane / kChunks, ld_p = lane % kChunks;
         if (wave == 0 && lane < kBiasBytes / 16) {
             const uint32_t n = uint32_t(lane) * 8 < g.n_valid ? uint32_t(lane) * 8 : 0u;
-            __builtin_amdgcn_global_load_lds((global_cptr)(g.bias + n), (lds_ptr)(smem + kBiasOffset + bias_slot * kBiasBytes), 16, 0, 0);
+            direct_load16<false>(g.bias + n, lds_address(smem) + kBiasOffset + bias_slot * kBiasBytes);
         }
         // The lane's source rows. The slot->token table was written earlier in the same launch,
         // possibly on another XCD: device-coherent loads, all in flight together (an index is clamped
@@ -348,7 +444,8 @@ struct Gemm16 {
     static __device__ __forceinline__ void mainloop(const Tile& t, Acc& acc, char* smem, Hook&& after_first_barrier) {
         const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
         const int wm = wave / WAVES_N, wn = wave % WAVES_N;
-        const int fr_row = lane & 31, fr_half = lane >> 5;
+        // a lane's share of an operand fragment: 16 bytes of row fr_row, the fr_part-th 8 values of the K step
+        const int fr_row = lane & (MI - 1), fr_part = lane / MI;
         if (rows_absent(t, __builtin_amdgcn_readfirstlane(wave) / WAVES_N)) {   // (a scalar condition: the branch holds barriers)
             // None of this wavefront's rows exist (an expert with few rows): it brings its share of
             // every slice into LDS at the same points of the same sequence of barriers as the others,
@@ -386,67 +483,104 @@ struct Gemm16 {
 #pragma unroll
             for (int mi = 0; mi < TM; ++mi)
 #pragma unroll
-                for (int v = 0; v < 16; ++v) acc[ni][mi][v] = 0.f;
-        // Fragment addresses inside a stage. Rows 32 apart share their swizzle, and K step ks only
-        // flips bits 5-6 of the chunk position, so one base per operand is enough: the address of
-        // block i at step ks is (base ^ (ks << 5)) + i * 32 rows.
+                for (int v = 0; v < int(sizeof(AccTile) / sizeof(float)); ++v) acc[ni][mi][v] = 0.f;
+        // Fragment addresses inside a stage. Rows MI apart share their swizzle, and K step ks only
+        // flips the upper bits of the chunk position (a step spans 2 chunks of 16 bytes with the
+        // 32-row tiles, 4 with the 16-row tiles), so one base per operand is enough: the address of
+        // block i at step ks is (base ^ (ks << kStepShift)) + i * MI rows.
+        constexpr int kStepShift = MI == 32 ? 5 : 6;
         const int rx = wm * WM + fr_row, rw = wn * WN + fr_row;
-        const int base_x = rx * kRowBytes + ((fr_half ^ swizzle(rx)) << 4);
-        const int base_w = kABytes + rw * kRowBytes + ((fr_half ^ swizzle(rw)) << 4);
+        const int base_x = rx * kRowBytes + ((fr_part ^ swizzle(rx)) << 4);
+        const int base_w = kABytes + rw * kRowBytes + ((fr_part ^ swizzle(rw)) << 4);
         // The operand fragments of K step ks+1 are read from LDS while the matrix core works on step ks.
-        vec8 fw[2][TN], fx[2][TM];
+        // 32-row tiles: two sets of fragments, fw[ks & 1] and fx[ks & 1]. 16-row tiles have twice as many
+        // fragments per step: the larger set (the `outer` one: x with tall wavefront tiles, w with wide
+        // ones) is walked in the outer loop of a step, each of its fragments serving NI instructions in
+        // a row and making way for its successor of the next step right behind them (one set of
+        // registers, fo); only the smaller set is kept twice (fi[ks & 1]).
+        constexpr bool kOuterX = TM >= TN;
+        constexpr int NO = kOuterX ? TM : TN, NI = kOuterX ? TN : TM;
+        static_assert(MI == 32 || (NI >= 2 && NO >= NI));
+        vec8 fw[2][MI == 32 ? TN : 1], fx[2][MI == 32 ? TM : 1];
+        vec8 fo[MI == 16 ? NO : 1], fi[2][MI == 16 ? NI : 1];
+        const int base_o = kOuterX ? base_x : base_w, base_i = kOuterX ? base_w : base_x;
         auto read_fragments = [&](const char* st, int ks) {
+            if constexpr (MI == 32) {
 #pragma unroll
-            for (int ni = 0; ni < TN; ++ni) fw[ks & 1][ni] = __builtin_bit_cast(vec8, load16(st + (base_w ^ (ks << 5)) + ni * 32 * kRowBytes));
+                for (int ni = 0; ni < TN; ++ni) fw[ks & 1][ni] = __builtin_bit_cast(vec8, load16(st + (base_w ^ (ks << kStepShift)) + ni * MI * kRowBytes));
 #pragma unroll
-            for (int mi = 0; mi < TM; ++mi) fx[ks & 1][mi] = __builtin_bit_cast(vec8, load16(st + (base_x ^ (ks << 5)) + mi * 32 * kRowBytes));
+                for (int mi = 0; mi < TM; ++mi) fx[ks & 1][mi] = __builtin_bit_cast(vec8, load16(st + (base_x ^ (ks << kStepShift)) + mi * MI * kRowBytes));
+            } else {
+#pragma unroll
+                for (int k = 0; k < NI; ++k) fi[ks & 1][k] = __builtin_bit_cast(vec8, load16(st + (base_i ^ (ks << kStepShift)) + k * MI * kRowBytes));
+#pragma unroll
+                for (int o = 0; o < NO; ++o) fo[o] = __builtin_bit_cast(vec8, load16(st + (base_o ^ (ks << kStepShift)) + o * MI * kRowBytes));
+            }
         };
         // Where one load of slice kn comes from and goes to (load li < LA: activation rows, else weight rows).
-        struct SliceLoads { char* sa; char* sb; uint32_t k0; };
+        struct SliceLoads { uint32_t sa, sb, k0; };
+        const uint32_t lds_wave = lds_address(smem) + 1024 * wave_index();
         auto loads_of = [&](uint32_t kn) {
             SliceLoads l;
-            l.sa = smem + stage_of(t, kn) * kStage;
+            l.sa = lds_wave + stage_of(t, kn) * kStage;
             l.sb = l.sa + kABytes;
             uint32_t slice = kn + t.k_first;
             slice = slice >= t.k_tiles ? slice - t.k_tiles : slice;
             l.k0 = slice * BK;
             return l;
         };
-        // K step ks in a pinned order: one matrix instruction, behind it one LDS read of step ks+1's
-        // fragments (the first TN + TM instructions) and, with LOADS, one global load of a later slice
-        // (loads load_base, load_base + 1, ... of it), and again. Issued as blocks - all reads, then all
+        // A quarter of a slice's matrix instructions (one K step with the 32-row tiles, half a K step
+        // with the 16-row tiles) in a pinned order: one matrix instruction, behind it one LDS read of the
+        // next K step's fragments (behind the first TN + TM instructions of a step) and, with LOADS, one
+        // global load of a later slice, and again. Issued as blocks - all reads, then all
         // matrix instructions - the two wavefronts of a SIMD took turns instead of overlapping, and a
         // slice's loads in a block in front of a K step held the matrix cores up (8 experts x 2560
         // rows, hidden size 4096, both projections: 3.80 ms in blocks, 3.49 with the reads interleaved,
         // 3.47 with the loads interleaved too; with operands resident in L2 3.49, 2.96 and 2.72).
-        // LOADS is a compile-time switch: a branch around matrix instructions makes the compiler keep
+        // The loads are a compile-time switch: a branch around matrix instructions makes the compiler keep
         // two copies of the accumulators.
-        // `first_tag`, `count_tag`: the K step carries the loads first .. first + count - 1 of the slice `l`
+        // `first_tag`, `count_tag`: the quarter carries the loads first .. first + count - 1 of the slice `l`
         // describes, evenly spaced behind its matrix instructions (count 0: none).
-        auto kstep = [&](const char* st, int ks, const SliceLoads& l, auto first_tag, auto count_tag) {
-            constexpr int FIRST = decltype(first_tag)::value, COUNT = decltype(count_tag)::value;
-            static_assert(COUNT <= TN * TM);
-            constexpr int kEvery = (TN * TM) / (COUNT > 0 ? COUNT : 1);
+        auto quarter = [&](const char* st, auto q_tag, const SliceLoads& l, auto first_tag, auto count_tag) {
+            constexpr int Q = decltype(q_tag)::value, FIRST = decltype(first_tag)::value, COUNT = decltype(count_tag)::value;
+            constexpr int kParts = kQuarters / kSteps;                 // quarters per K step
+            constexpr int ks = Q / kParts, part = Q % kParts;
+            static_assert(COUNT <= kPerQuarter);
+            constexpr int kEvery = kPerQuarter / (COUNT > 0 ? COUNT : 1);
 #pragma unroll
-            for (int i = 0; i < TN * TM; ++i) {
+            for (int j = 0; j < kPerQuarter; ++j) {
                 __builtin_amdgcn_sched_barrier(0);
-                const int ni = i / TM, mi = i % TM;
-                acc[ni][mi] = Elem16<E>::mfma32(fw[ks & 1][ni], fx[ks & 1][mi], acc[ni][mi]);
-                if (ks + 1 < kSteps) {
-                    const int nb = (ks + 1) & 1;
-                    if (i < TN) fw[nb][i] = __builtin_bit_cast(vec8, load16(st + (base_w ^ ((ks + 1) << 5)) + i * 32 * kRowBytes));
-                    else if (i < TN + TM) fx[nb][i - TN] = __builtin_bit_cast(vec8, load16(st + (base_x ^ ((ks + 1) << 5)) + (i - TN) * 32 * kRowBytes));
+                const int i = part * kPerQuarter + j;                  // the step's i-th matrix instruction
+                if constexpr (MI == 32) {
+                    const int ni = i / TM, mi = i % TM;
+                    acc[ni][mi] = Elem16<E>::mfma32(fw[ks & 1][ni], fx[ks & 1][mi], acc[ni][mi]);
+                    if (ks + 1 < kSteps) {
+                        const int nb = (ks + 1) & 1;
+                        if (i < TN) fw[nb][i] = __builtin_bit_cast(vec8, load16(st + (base_w ^ ((ks + 1) << kStepShift)) + i * MI * kRowBytes));
+                        else if (i < TN + TM) fx[nb][i - TN] = __builtin_bit_cast(vec8, load16(st + (base_x ^ ((ks + 1) << kStepShift)) + (i - TN) * MI * kRowBytes));
+                    }
+                } else {
+                    const int o = i / NI, k = i % NI;
+                    if constexpr (kOuterX) acc[k][o] = Elem16<E>::mfma16(fi[ks & 1][k], fo[o], acc[k][o]);
+                    else acc[o][k] = Elem16<E>::mfma16(fo[o], fi[ks & 1][k], acc[o][k]);
+                    if (ks + 1 < kSteps) {
+                        // behind the last instruction that uses fo[o]: its successor; behind the first
+                        // instructions of the first NI outer rounds: the inner set of the next step
+                        if (k == NI - 1) fo[o] = __builtin_bit_cast(vec8, load16(st + (base_o ^ ((ks + 1) << kStepShift)) + o * MI * kRowBytes));
+                        else if (k == 0 && o < NI) fi[(ks + 1) & 1][o] = __builtin_bit_cast(vec8, load16(st + (base_i ^ ((ks + 1) << kStepShift)) + o * MI * kRowBytes));
+                    }
                 }
                 if constexpr (COUNT > 0) {
-                    if (i % kEvery == 0 && i / kEvery < COUNT) issue_one(t, l.sa, l.sb, l.k0, FIRST + i / kEvery);
+                    if (j % kEvery == 0 && j / kEvery < COUNT) issue_one(t, l.sa, l.sb, l.k0, FIRST + j / kEvery);
                 }
             }
             __builtin_amdgcn_sched_barrier(0);
         };
-        static_assert(TN + TM <= TN * TM, "a K step has a matrix instruction for every fragment read");
+        using Q0 = std::integral_constant<int, 0>; using Q1 = std::integral_constant<int, 1>;
+        using Q2 = std::integral_constant<int, 2>; using Q3 = std::integral_constant<int, 3>;
+        static_assert(MI == 16 || TN + TM <= kPerQuarter, "the first quarter of a K step has a matrix instruction for every fragment read");
         if constexpr (AHEAD2) {
-            static_assert(LA + LB <= TN * TM, "the loads of a slice fit behind the matrix instructions of one K step");
-            static_assert(kSteps == 4);
+            static_assert(LA + LB <= kPerQuarter, "the loads of a slice fit behind the matrix instructions of one quarter");
             constexpr int N0 = spread_count(0), N1 = spread_count(1), N2 = spread_count(2), N3 = spread_count(3);
             // Slice 0 was requested by begin(). Every wavefront has left the previous tile's epilogue,
             // which staged its output in the stage slice 1 goes to: its first loads go out here, the
@@ -467,9 +601,9 @@ struct Gemm16 {
                 const char* st = smem + stage_of(t, kt) * kStage;
                 read_fragments(st, 0);
                 const SliceLoads l1 = NEXT ? loads_of(kt + 1) : SliceLoads{};
-                kstep(st, 0, l1, std::integral_constant<int, N0>{}, std::integral_constant<int, NEXT ? N1 : 0>{});
-                kstep(st, 1, l1, std::integral_constant<int, N0 + N1>{}, std::integral_constant<int, NEXT ? N2 : 0>{});
-                kstep(st, 2, l1, std::integral_constant<int, N0 + N1 + N2>{}, std::integral_constant<int, NEXT ? N3 : 0>{});
+                quarter(st, Q0{}, l1, std::integral_constant<int, N0>{}, std::integral_constant<int, NEXT ? N1 : 0>{});
+                quarter(st, Q1{}, l1, std::integral_constant<int, N0 + N1>{}, std::integral_constant<int, NEXT ? N2 : 0>{});
+                quarter(st, Q2{}, l1, std::integral_constant<int, N0 + N1 + N2>{}, std::integral_constant<int, NEXT ? N3 : 0>{});
                 if constexpr (NEXT2) {
                     // this wavefront's last reads of the stage have returned; once that holds for every
                     // wavefront the stage takes slice kt+2
@@ -477,14 +611,14 @@ struct Gemm16 {
                     asm volatile("s_barrier" ::: "memory");
                 }
                 const SliceLoads l2 = NEXT2 ? loads_of(kt + 2) : SliceLoads{};
-                kstep(st, 3, l2, std::integral_constant<int, 0>{}, std::integral_constant<int, NEXT2 ? N0 : 0>{});
+                quarter(st, Q3{}, l2, std::integral_constant<int, 0>{}, std::integral_constant<int, NEXT2 ? N0 : 0>{});
             };
             const uint32_t ahead = t.k_tiles >= 2 ? t.k_tiles - 2 : 0u;   // slices that request slice kt+2
             for (uint32_t kt = 0; kt < ahead; ++kt) slice(kt, std::true_type{}, std::true_type{});
             if (t.k_tiles >= 2) slice(t.k_tiles - 2, std::true_type{}, std::false_type{});
             slice(t.k_tiles - 1, std::false_type{}, std::false_type{});
         } else {
-            static_assert(LA + LB <= kSteps * TN * TM, "the loads of a slice fit behind the matrix instructions of a slice");
+            static_assert(LA + LB <= kQuarters * kPerQuarter, "the loads of a slice fit behind the matrix instructions of a slice");
             auto top = [&](uint32_t kt) {
                 // This wavefront's loads of slice kt are complete once only those of the later slices
                 // already issued (STAGES-2 of them, fewer at the end of the tile) are outstanding.
@@ -497,16 +631,16 @@ struct Gemm16 {
                 asm volatile("s_barrier" ::: "memory");
                 if (kt == 0) after_first_barrier();
             };
-            // K step ks carries the loads ks * TN * TM ... of the slice STAGES-1 ahead, one behind each
+            // Quarter q carries the loads q * kPerQuarter ... of the slice STAGES-1 ahead, one behind each
             // matrix instruction, until they run out (sharing them out evenly over the four K steps,
             // which three stages would allow, changes nothing where it was measured: 2.93 against
             // 2.92 ms per forward at the 256-expert top-8 shape, which is bound by HBM)
             auto ksteps = [&](const char* st, const SliceLoads& l, auto loads_tag) {
-                static_for<kSteps>([&](auto ks_tag) {
-                    constexpr int ks = decltype(ks_tag)::value;
-                    constexpr int left = LA + LB - ks * TN * TM;
-                    constexpr int count = !decltype(loads_tag)::value || left <= 0 ? 0 : (left < TN * TM ? left : TN * TM);
-                    kstep(st, ks, l, std::integral_constant<int, ks * TN * TM>{}, std::integral_constant<int, count>{});
+                static_for<kQuarters>([&](auto q_tag) {
+                    constexpr int q = decltype(q_tag)::value;
+                    constexpr int left = LA + LB - q * kPerQuarter;
+                    constexpr int count = !decltype(loads_tag)::value || left <= 0 ? 0 : (left < kPerQuarter ? left : kPerQuarter);
+                    quarter(st, q_tag, l, std::integral_constant<int, q * kPerQuarter>{}, std::integral_constant<int, count>{});
                 });
             };
             const uint32_t ahead = t.k_tiles >= uint32_t(STAGES - 1) ? t.k_tiles - (STAGES - 1) : 0u;   // slices that request a later one
@@ -547,6 +681,7 @@ struct Gemm16 {
     // 4 KB of its own in the stage of the last slice (rows of 128 bytes, chunk c of row r at position
     // c ^ ((r >> 1) & 7)) and stores whole 128-byte lines.
     static __device__ __forceinline__ void finish_partial(const Tile& t, Acc& acc, char* smem, float* out, uint32_t ldo) {
+        static_assert(MI == 32, "written for the accumulator layout of the 32 x 32 tiles");
         const uint32_t tid = local_tid();
         const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
         const int wm = wave / WAVES_N, wn = wave % WAVES_N;

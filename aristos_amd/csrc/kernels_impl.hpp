@@ -71,10 +71,16 @@ constexpr int kXcds = 8;
 #ifndef KLEOS_TUNE_MIXED_HEIGHTS
 #define KLEOS_TUNE_MIXED_HEIGHTS 1   // variant 2: 128-row tiles for last row blocks of at most 128 rows
 #endif
+#ifndef KLEOS_TUNE_MI
+#define KLEOS_TUNE_MI 16           // matrix-core tile of the expert GEMM: 16 (16x16x32 instructions) or 32 (32x32x16)
+#endif
+#ifndef KLEOS_TUNE_MI_V0
+#define KLEOS_TUNE_MI_V0 16        // the same for variant 0 (switchable apart: its tiles are the ones bound by their loads)
+#endif
 template <typename E, int V>
-using GemmCfg = std::conditional_t<V == 0, Gemm16<E, 256, 256, 4, 2, 64, 2, true, true, KLEOS_TUNE_V0_SPREAD>,
-                std::conditional_t<V == 1, Gemm16<E, 128, 256, 2, 4, 64, 3, true, false>,
-                                   Gemm16<E, 256, 256, 2, 4, 64, 2, false, (KLEOS_TUNE_V2_SPREAD >= 0), (KLEOS_TUNE_V2_SPREAD >= 0 ? KLEOS_TUNE_V2_SPREAD : 0)>>>;
+using GemmCfg = std::conditional_t<V == 0, Gemm16<E, 256, 256, 4, 2, 64, 2, true, true, KLEOS_TUNE_V0_SPREAD, KLEOS_TUNE_MI_V0>,
+                std::conditional_t<V == 1, Gemm16<E, 128, 256, 2, 4, 64, 3, true, false, 0, KLEOS_TUNE_MI>,
+                                   Gemm16<E, 256, 256, 2, 4, 64, 2, false, (KLEOS_TUNE_V2_SPREAD >= 0), (KLEOS_TUNE_V2_SPREAD >= 0 ? KLEOS_TUNE_V2_SPREAD : 0), KLEOS_TUNE_MI>>>;
 // Layers of variant 2 mix two tile heights inside one launch: the last row block of an expert, when
 // it holds at most 128 rows, goes to a 128 x 256 tile (three stages, loads two slices ahead of the
 // slice being worked on) instead of a 256-row tile whose lower half would multiply rows that do
@@ -82,7 +88,7 @@ using GemmCfg = std::conditional_t<V == 0, Gemm16<E, 256, 256, 4, 2, 64, 2, true
 // differs. (The K order of every output element is the same in both tiles: same slices, same
 // matrix instruction, so which tile computed a row does not show in its bits.)
 template <typename E, int V>
-using NarrowCfg = Gemm16<E, 128, 256, 2, 4, 64, 3, false, false>;
+using NarrowCfg = Gemm16<E, 128, 256, 2, 4, 64, 3, false, false, 0, KLEOS_TUNE_MI>;
 template <typename G> struct TypeTag { using type = G; };   // a type handed to a generic lambda
 template <typename T, int V> constexpr bool kMixedHeights = sizeof(T) == 2 && V == 2 && KLEOS_TUNE_MIXED_HEIGHTS != 0;
 constexpr uint32_t kNarrowTileRows = 128;

@@ -1,6 +1,7 @@
 """Benchmark of the fused MoE-layer forward on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu-baseline]
+                    [--power-seconds S] [--zero-expert-weights] [--calib-gemm M,N,K]
 
 A step is one forward of the layer (one persistent kernel launch) over one batch of synthetic
 tokens already resident in HBM. The per-phase figures are measured first, with launch counts of
@@ -10,7 +11,9 @@ loses them within milliseconds of idling); then come the timed region proper: `w
 forwards and exactly `steps` forwards between two readings of the wall clock. Prints one JSON line: latency per forward, the roofline of the
 launch (the workload's arithmetic intensity decides which roof binds: algorithmic bytes / event-timed
 duration against HBM peak, with the matrix-core fraction beside it), per-phase figures from the
-phased mode, and the CPU oracle timed on this box's host cores as a baseline.
+phased mode, and the CPU oracle timed on this box's host cores as a baseline. After the timed region
+the forwards keep running for `--power-seconds` while a thread reads the socket power (`power`): all
+of these workloads hold the package at its 1400 W cap, and so does the vendor's GEMM (`--calib-gemm`).
 """
 from __future__ import annotations
 
@@ -58,6 +61,102 @@ def measured_traffic(workload: str):
     return float(m.group(1)) * 1e9, bool(fp and fp.group(1) == source_fingerprint())
 
 
+class PowerSampler:
+    """Socket power while a load runs, read from the amdgpu hwmon node (power1_input, microwatts)
+    every 0.2 s by a thread. MI355X caps the package at power1_cap (1400 W); a load that sits at the
+    cap runs at whatever clocks that power buys, so its duration follows the energy it needs."""
+
+    def __init__(self):
+        import glob
+        nodes = sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_input"))
+        self.path = nodes[0] if nodes else None
+        self.samples, self._stop, self._thread = [], False, None
+
+    @staticmethod
+    def _read(path):
+        try:
+            with open(path) as f:
+                return int(f.read().strip()) / 1e6
+        except (OSError, ValueError):
+            return None
+
+    def cap_w(self):
+        return self._read(self.path.replace("power1_input", "power1_cap")) if self.path else None
+
+    def start(self):
+        import threading
+        if not self.path:
+            return
+
+        def run():
+            while not self._stop:
+                v = self._read(self.path)
+                if v is not None:
+                    self.samples.append((time.perf_counter(), v))
+                time.sleep(0.2)
+        self._thread = threading.Thread(target=run, daemon=True)
+        self._thread.start()
+
+    def stop(self, since: float):
+        """Mean and maximum of the samples taken after `since` (perf_counter seconds)."""
+        self._stop = True
+        if self._thread:
+            self._thread.join()
+        vals = [v for t, v in self.samples if t >= since]
+        if not vals:
+            return None
+        return {"mean_w": round(sum(vals) / len(vals), 1), "max_w": round(max(vals), 1), "samples": len(vals),
+                "cap_w": self.cap_w(), "source": self.path}
+
+
+def sustained_power(seconds: float, launch_some) -> dict | None:
+    """Runs `launch_some()` (a few dozen milliseconds of back-to-back work that ends synchronised)
+    for `seconds` and returns the socket power over all but the first 1.5 s."""
+    ps = PowerSampler()
+    ps.start()
+    t0 = time.perf_counter()
+    n = 0
+    while time.perf_counter() - t0 < seconds:
+        launch_some()
+        n += 1
+    out = ps.stop(t0 + 1.5)
+    if out is not None:
+        out["seconds"] = round(time.perf_counter() - t0, 2)
+    return out
+
+
+def vendor_gemm_calibration(shape: str, seconds: float, zero_a: bool) -> int:
+    """`--calib-gemm M,N,K`: the vendor's bf16 GEMM (torch `a @ b.T`, hipBLASLt) on random operands
+    of one projection's shape, looped for `seconds`: TFLOP/s and socket power. What another kernel
+    reaches on this box, this data and this power cap; not part of the library."""
+    import torch
+    M, N, K = (int(v) for v in shape.split(","))
+    a = torch.randn(M, K, device="cuda", dtype=torch.bfloat16) * 0.5
+    b = torch.randn(N, K, device="cuda", dtype=torch.bfloat16) * 0.02
+    if zero_a:
+        a.zero_()
+    c = torch.empty(M, N, device="cuda", dtype=torch.bfloat16)
+    torch.matmul(a, b.T, out=c)
+    torch.cuda.synchronize()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    reps = max(1, int(0.05 / (2.0 * M * N * K / 1.2e15)))
+    rates = []
+
+    def some():
+        ev0.record()
+        for _ in range(reps):
+            torch.matmul(a, b.T, out=c)
+        ev1.record()
+        torch.cuda.synchronize()
+        rates.append(2.0 * M * N * K * reps / (ev0.elapsed_time(ev1) * 1e-3) / 1e12)
+    power = sustained_power(max(3.0, seconds), some)
+    tail = rates[len(rates) // 2:]
+    print(json.dumps({"calibration": "vendor bf16 GEMM (torch matmul, a @ b.T)", "M": M, "N": N, "K": K,
+                      "a_zeroed": zero_a, "tflops": round(sum(tail) / len(tail), 1),
+                      "mfma_frac": round(sum(tail) / len(tail) / PEAK_BF16_TFLOPS, 4), "power": power}))
+    return 0
+
+
 PHASED_SKIP, FUSED_SKIP, REHEARSALS = 8, 32, 3
 
 
@@ -90,6 +189,16 @@ def main() -> int:
     ap.add_argument("--calib-copy-mib", type=int, default=0,
                     help="also run one device-to-device copy of this many MiB before the timed region "
                          "(a kernel of known traffic to scale rocprofv3 FETCH_SIZE / WRITE_SIZE by)")
+    ap.add_argument("--power-seconds", type=float, default=4.0,
+                    help="after the timed region, keep launching forwards for this long and report the socket "
+                         "power over that time (0: skip)")
+    ap.add_argument("--zero-expert-weights", action="store_true",
+                    help="power probe, not the metric: the expert weights are zeroed, so that the same kernel "
+                         "with the same schedule and memory traffic multiplies zeros")
+    ap.add_argument("--calib-gemm", default="",
+                    help="M,N,K: instead of the layer, loop the vendor's bf16 GEMM of that shape for "
+                         "--power-seconds and report its TFLOP/s and socket power (add --zero-expert-weights "
+                         "to zero its first operand)")
     ap.add_argument("--print-fingerprint", action="store_true",
                     help="print the fingerprint of the library sources (recorded in the counter summaries) and exit")
     args = ap.parse_args()
@@ -112,8 +221,12 @@ def main() -> int:
         print("bench.py needs a GPU", file=sys.stderr)
         return 2
     torch.cuda.set_device(0)
+    if args.calib_gemm:
+        return vendor_gemm_calibration(args.calib_gemm, args.power_seconds, args.zero_expert_weights)
     w = synth.WORKLOADS[args.workload]
     iP, d = synth.make_inputs(w, seed=args.seed, device="cuda")
+    if args.zero_expert_weights:
+        iP.view(-1)[d.off_w_up:d.off_w_up + 2 * d.E * d.I * d.H].zero_()
     torch.cuda.synchronize()
     bf16 = d.elem_bytes == 2
 
@@ -166,6 +279,16 @@ def main() -> int:
         ka.moe.forward_host_bench(iP, oP, skip=0, trials=8)
         fused_ph = ka.moe.phase_times()
         sched = ka.moe.scheduler_stats()
+        # socket power under the same load, kept up for a few seconds, and what a forward takes then
+        power = None
+        if args.power_seconds > 0:
+            per_call = max(8, int(0.05 / max(wall_ms * 1e-3, 1e-6)))
+            seen = []
+            power = sustained_power(args.power_seconds, lambda: seen.append(
+                (time.perf_counter(), ka.moe.forward_host_bench(iP, oP, skip=0, trials=per_call))))
+            if power is not None and seen:
+                late = [ms for t, ms in seen if t >= seen[0][0] + 1.5] or [ms for _, ms in seen]
+                power["sustained_ms_per_step"] = round(sum(late) / len(late), 5)
         schedule = "static" if ka.moe.schedule_taken() == ka.SCHEDULE_STATIC else "dynamic"
         views = ka.moe.debug_views(d)
         kept = int(np.minimum(views["expert_count"].astype(np.int64), d.kept_capacity).sum())
@@ -229,7 +352,7 @@ def main() -> int:
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "bf16" if bf16 else "f32",
-        "data": "synthetic",
+        "data": "synthetic" if not args.zero_expert_weights else "synthetic, expert weights zeroed (power probe: not the metric)",
         "config": {"workload": f"{w.name}: {w.note}", "S": d.S, "H": d.H, "I": d.I, "E": d.E, "top_k": d.k,
                    "capacity_factor": w.config.capacity_factor, "EC": d.EC, "kept_pairs": kept,
                    "dropped_pairs": dropped, "hottest_expert_vs_mean": round(hottest, 2),
@@ -238,6 +361,7 @@ def main() -> int:
         "tokens_per_s": round(d.S / (wall_ms * 1e-3), 1),
         "event_ms_per_step": round(ev_ms, 5),
         "roofline": roofline(flops_layer, hbm_bytes, ev_ms, peak, traffic_bytes, traffic_current, experts),
+        "power": power,
         "fused_phases": fused_phases,
         "phased_mode": phases,
         "cpu_baseline": cpu,

@@ -49,3 +49,23 @@ def test_the_json_line_says_what_ran_before_the_timed_region():
     assert rec["prewarm_detail"]["rehearsal_passes"] == 3 and len(rec["pass_ms_per_step"]) == 4
     src = open(os.path.join(ROOT, "bench.py")).read()
     assert "**prewarm_protocol(args.steps, args.warmup, pass_ms)" in src   # the keys reach the printed line
+
+
+def test_power_sampler_reads_a_hwmon_node_and_reports_none_without_one(tmp_path, monkeypatch):
+    """The socket-power figure comes from power1_input (microwatts) of the amdgpu hwmon node; a box
+    without the node gets `power: null`, never a made-up number."""
+    assert bench.sustained_power(0.3, lambda: None) is None or "mean_w" in bench.sustained_power(0.3, lambda: None)
+    node = tmp_path / "power1_input"
+    node.write_text("1399000000\n")
+    (tmp_path / "power1_cap").write_text("1400000000\n")
+    import glob
+    monkeypatch.setattr(glob, "glob", lambda pattern: [str(node)])
+    import time
+    t0 = time.perf_counter()
+    ps = bench.PowerSampler()
+    ps.start()
+    time.sleep(0.5)
+    out = ps.stop(t0)
+    assert out["mean_w"] == 1399.0 and out["max_w"] == 1399.0 and out["cap_w"] == 1400.0 and out["samples"] >= 2
+    src = open(os.path.join(ROOT, "bench.py")).read()
+    assert '"power": power' in src
