@@ -269,6 +269,9 @@ __device__ __forceinline__ void static_for(F&& f) {
 // late (4.07 ms at the shape above); one barrier per slice instead of two (the barrier in front of the
 // last K step also standing for "the next slice has landed", its first fragments read behind that K
 // step's matrix instructions) loses the lead time it needs: 3.98 ms.
+#ifndef KLEOS_GEMM_BLOCK_SKIP
+#define KLEOS_GEMM_BLOCK_SKIP 1
+#endif
 // MI: the matrix-core tile. 32: 32x32x16 instructions (16 values of K each, 16 accumulator registers);
 // 16: 16x16x32 instructions (32 values of K, 4 accumulator registers). The smaller tile reads and
 // writes half as many accumulator registers per multiply-add and draws less power for the same work
@@ -295,6 +298,10 @@ struct Gemm16 {
     static constexpr int kLoadsPerSlice = LA + LB;                 // per wavefront
     static constexpr int kSliceK = BK;                             // values of K per slice
     static constexpr int kSteps = BK / KI;                         // K steps per slice
+    // 16-row tiles, wavefront tiles of four of them in height: a wavefront leaves out the blocks of 16
+    // rows that hold no rows of the tile (64-expert shape with skewed routing: the experts' 13 039 rows
+    // take the matrix instructions of 13 424 rows that way, of 14 656 with whole wavefronts left out only)
+    static constexpr bool kBlockSkip = KLEOS_GEMM_BLOCK_SKIP != 0 && MI == 16 && TM == 4;
     static constexpr int kQuarters = 4;                            // a slice's matrix instructions in four equal runs
     static constexpr int kPerQuarter = TN * TM * kSteps / kQuarters;
     static constexpr int kPanelRows = kEpiloguePanelRows;          // epilogue staging: 32 rows x 64 columns per wavefront
@@ -305,10 +312,19 @@ struct Gemm16 {
         switch (SPREAD) {
             case 1: return i < 2 ? L / 2 : 0;                                                       // 4 4 0 0
             case 2: return i == 0 || i == 1 ? (3 * L) / 8 : (i == 2 ? L - 2 * ((3 * L) / 8) : 0);   // 3 3 2 0
+#ifdef KLEOS_X_SPREADS
+            case 3: return L / 4;                                                                   // 2 2 2 2
+            case 4: return i == 0 ? L / 4 : (i == 1 ? (3 * L) / 4 : 0);                             // 2 6 0 0
+            case 5: return i == 0 ? (3 * L) / 4 : (i == 1 ? L / 4 : 0);                             // 6 2 0 0
+            case 6: return i == 0 ? L / 2 : (i == 1 || i == 2 ? L / 4 : 0);                         // 4 2 2 0
+            case 7: return i == 1 ? L / 2 : (i == 0 || i == 2 ? L / 4 : 0);                         // 2 4 2 0
+#endif
             default: return i == 0 ? L : 0;                                                         // all at once
         }
     }
+#ifndef KLEOS_X_SPREADS
     static_assert(SPREAD >= 0 && SPREAD <= 2);
+#endif
     static_assert(SPREAD == 0 || (AHEAD2 && (LA + LB) % 8 == 0));
     static_assert(spread_count(0) + spread_count(1) + spread_count(2) + spread_count(3) == LA + LB);
     static_assert(BK == 32 || BK == 64);
@@ -501,6 +517,12 @@ struct Gemm16 {
         constexpr bool kOuterX = TM >= TN;
         constexpr int NO = kOuterX ? TM : TN, NI = kOuterX ? TN : TM;
         static_assert(MI == 32 || (NI >= 2 && NO >= NI));
+        // XB: how many of the wavefront's TM blocks of MI rows hold rows of the tile. The blocks behind
+        // them are left out of the fragment reads and the matrix instructions (with the 16-row tiles, in
+        // the configurations that take the trouble: kBlockSkip); their accumulators are never stored.
+        auto body = [&](auto xb_tag) {
+        constexpr int XB = decltype(xb_tag)::value;
+        auto x_block_used = [](int mi) { return mi < XB; };
         vec8 fw[2][MI == 32 ? TN : 1], fx[2][MI == 32 ? TM : 1];
         vec8 fo[MI == 16 ? NO : 1], fi[2][MI == 16 ? NI : 1];
         const int base_o = kOuterX ? base_x : base_w, base_i = kOuterX ? base_w : base_x;
@@ -512,9 +534,11 @@ struct Gemm16 {
                 for (int mi = 0; mi < TM; ++mi) fx[ks & 1][mi] = __builtin_bit_cast(vec8, load16(st + (base_x ^ (ks << kStepShift)) + mi * MI * kRowBytes));
             } else {
 #pragma unroll
-                for (int k = 0; k < NI; ++k) fi[ks & 1][k] = __builtin_bit_cast(vec8, load16(st + (base_i ^ (ks << kStepShift)) + k * MI * kRowBytes));
+                for (int k = 0; k < NI; ++k)
+                    if (kOuterX || x_block_used(k)) fi[ks & 1][k] = __builtin_bit_cast(vec8, load16(st + (base_i ^ (ks << kStepShift)) + k * MI * kRowBytes));
 #pragma unroll
-                for (int o = 0; o < NO; ++o) fo[o] = __builtin_bit_cast(vec8, load16(st + (base_o ^ (ks << kStepShift)) + o * MI * kRowBytes));
+                for (int o = 0; o < NO; ++o)
+                    if (!kOuterX || x_block_used(o)) fo[o] = __builtin_bit_cast(vec8, load16(st + (base_o ^ (ks << kStepShift)) + o * MI * kRowBytes));
             }
         };
         // Where one load of slice kn comes from and goes to (load li < LA: activation rows, else weight rows).
@@ -561,13 +585,18 @@ struct Gemm16 {
                     }
                 } else {
                     const int o = i / NI, k = i % NI;
-                    if constexpr (kOuterX) acc[k][o] = Elem16<E>::mfma16(fi[ks & 1][k], fo[o], acc[k][o]);
-                    else acc[o][k] = Elem16<E>::mfma16(fo[o], fi[ks & 1][k], acc[o][k]);
+                    if (x_block_used(kOuterX ? o : k)) {   // (folds at compile time: o and k are unrolled)
+                        if constexpr (kOuterX) acc[k][o] = Elem16<E>::mfma16(fi[ks & 1][k], fo[o], acc[k][o]);
+                        else acc[o][k] = Elem16<E>::mfma16(fo[o], fi[ks & 1][k], acc[o][k]);
+                    }
                     if (ks + 1 < kSteps) {
                         // behind the last instruction that uses fo[o]: its successor; behind the first
                         // instructions of the first NI outer rounds: the inner set of the next step
-                        if (k == NI - 1) fo[o] = __builtin_bit_cast(vec8, load16(st + (base_o ^ ((ks + 1) << kStepShift)) + o * MI * kRowBytes));
-                        else if (k == 0 && o < NI) fi[(ks + 1) & 1][o] = __builtin_bit_cast(vec8, load16(st + (base_i ^ ((ks + 1) << kStepShift)) + o * MI * kRowBytes));
+                        if (k == NI - 1) {
+                            if (!kOuterX || x_block_used(o)) fo[o] = __builtin_bit_cast(vec8, load16(st + (base_o ^ ((ks + 1) << kStepShift)) + o * MI * kRowBytes));
+                        } else if (k == 0 && o < NI) {
+                            if (kOuterX || x_block_used(o)) fi[(ks + 1) & 1][o] = __builtin_bit_cast(vec8, load16(st + (base_i ^ ((ks + 1) << kStepShift)) + o * MI * kRowBytes));
+                        }
                     }
                 }
                 if constexpr (COUNT > 0) {
@@ -656,6 +685,21 @@ struct Gemm16 {
                 read_fragments(st, 0);
                 ksteps(st, SliceLoads{}, std::false_type{});
             }
+        }
+        };   // body
+        if constexpr (kBlockSkip) {
+            // (the same in all lanes of a wavefront; every version goes through the same barriers)
+            const int rows_here = int(t.m_valid) - __builtin_amdgcn_readfirstlane(wave) / WAVES_N * WM;
+            const int used = rows_here >= WM ? TM : (rows_here <= MI ? 1 : (rows_here + MI - 1) / MI);
+            static_assert(TM == 4);
+            switch (used) {
+                case 1: body(std::integral_constant<int, 1>{}); break;
+                case 2: body(std::integral_constant<int, 2>{}); break;
+                case 3: body(std::integral_constant<int, 3>{}); break;
+                default: body(std::integral_constant<int, 4>{}); break;
+            }
+        } else {
+            body(std::integral_constant<int, TM>{});
         }
     }
 

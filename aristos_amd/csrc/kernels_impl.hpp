@@ -36,7 +36,11 @@ constexpr int kXcds = 8;
 // Expert GEMM configuration of the bf16 / fp16 path: 256 x 256 tile (an expert's whole capacity of
 // 256 rows at the headline shape, so its weights stream from HBM exactly once), 4 x 2 wavefronts of
 // 64 x 128 (two per SIMD), K slices of 64 (whole 128-byte lines of every row) through two 64 KB
-// stages, loads two slices ahead, a slice's loads shared out 3 + 3 + 2 over three K steps.
+// stages, loads two slices ahead, a slice's loads shared out 4 + 4 over two quarters of a slice's
+// matrix instructions, which are the 16x16x32 ones (see Gemm16: they draw less power, and power is
+// what bounds these kernels: 292 against 298 us per forward at the headline shape with 32x32x16,
+// 3.16 against 3.28 ms at the 8-expert shape with hidden size 4096; with them 4 + 4 beats 3 + 3 + 2,
+// which was the better split for the 32x32x16 instructions, 291 against 298 us).
 // (Measured against it on MI355X, none faster: K slices of 32 through four stages, 2 x 2 wavefronts
 // of 128 x 128 with the accumulators in AGPRs, weight slices of 64 through three slots with
 // activation half slices of 32 through three, the 128 x 256 tile of variant 1. 2 x 4 wavefronts
@@ -55,9 +59,9 @@ constexpr int kXcds = 8;
 // Variants 0 and 1 load their weight rows non-temporally (headline 378 against 390 us per forward,
 // the 16-expert shape 192 against 196, the 256-expert shape 3.43 against 3.48 ms); variant 2, whose
 // weight tiles are shared by eight workgroups and more, does not (4.06 against 4.01 ms with it).
-// (The three choices below can be overridden on the compiler's command line for measurements.)
+// (The choices below can be overridden on the compiler's command line for measurements.)
 #ifndef KLEOS_TUNE_V0_SPREAD
-#define KLEOS_TUNE_V0_SPREAD 2       // variant 0: loads of a slice issued 3 + 3 + 2 over three K steps
+#define KLEOS_TUNE_V0_SPREAD 1       // variant 0: loads of a slice issued 4 + 4 over two quarters of a slice (2: 3 + 3 + 2)
 #endif
 #ifndef KLEOS_TUNE_V2_SPREAD
 #define KLEOS_TUNE_V2_SPREAD 1       // variant 2: two slices ahead, 4 + 4 over two K steps; -1: one slice ahead
