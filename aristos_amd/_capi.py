@@ -60,6 +60,7 @@ SYMBOLS = {
     "kleos_static_scratch_status": (C.c_int, [C.c_void_p]),
     "kleos_debug_static_scratch_expiry": (C.c_int, [C.c_ulonglong, C.c_uint32]),
     "kleos_debug_map_hip_error": (C.c_int, [C.c_int]),
+    "kleos_debug_mfma_probe": (C.c_int, [C.c_int, C.c_uint32, C.c_int, C.POINTER(C.c_float), C.POINTER(C.c_double)]),
     "kleos_stream_synchronize": (C.c_int, []),
     "kleos_stream": (C.c_void_p, []),
     "kleos_set_mode": (C.c_int, [C.c_int]),

@@ -386,6 +386,41 @@ extern "C" int kleos_debug_map_hip_error(int hip_error) {
     return KLEOS_OK;
 }
 
+// The matrix-instruction probe keeps 16 MB of operand patterns and its timing events on the current
+// device until the process ends (a measurement aid: nothing of the layer touches them).
+extern "C" int kleos_debug_mfma_probe(int tile, uint32_t iterations, int zero_operands, float* ms, double* flop) {
+    static std::mutex mu;
+    static uint32_t* data = nullptr;
+    static float* sink = nullptr;
+    static int filled_zero = -1, cus = 0;
+    static hipEvent_t ev[2];
+    if (!ms || !flop) return fail(KLEOS_EINVAL, "kleos_debug_mfma_probe: null argument");
+    if ((tile != 16 && tile != 32) || iterations == 0)
+        return fail(KLEOS_EINVAL, "kleos_debug_mfma_probe: tile must be 16 or 32 and iterations positive");
+    std::lock_guard<std::mutex> lock(mu);
+    if (!data) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        KLEOS_HIP(hipGetDevice(&dev));
+        KLEOS_HIP(hipGetDeviceProperties(&prop, dev));
+        cus = prop.multiProcessorCount;
+        KLEOS_HIP(hipMalloc(&sink, sizeof(float)));
+        KLEOS_HIP(hipEventCreate(&ev[0]));
+        KLEOS_HIP(hipEventCreate(&ev[1]));
+        KLEOS_HIP(hipMalloc(&data, kMfmaProbeWords * sizeof(uint32_t)));
+    }
+    if (filled_zero != (zero_operands != 0)) {
+        KLEOS_HIP(launch_mfma_probe_fill(data, kMfmaProbeWords, zero_operands != 0, nullptr));
+        filled_zero = zero_operands != 0;
+    }
+    KLEOS_HIP(hipEventRecord(ev[0], nullptr));
+    KLEOS_HIP(launch_mfma_probe(tile, iterations, data, sink, cus, flop, nullptr));
+    KLEOS_HIP(hipEventRecord(ev[1], nullptr));
+    KLEOS_HIP(hipEventSynchronize(ev[1]));
+    KLEOS_HIP(hipEventElapsedTime(ms, ev[0], ev[1]));
+    return KLEOS_OK;
+}
+
 extern "C" int kleos_initialize_cfg(const kleos_config_t* user_cfg) {
     if (!user_cfg) return fail(KLEOS_EINVAL, "kleos_initialize_cfg: null config");
     if (g_ctx) return fail(KLEOS_ESTATE, "Already Initialized");   // bootstrap.cuh:537

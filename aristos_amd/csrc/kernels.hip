@@ -92,4 +92,71 @@ hipError_t launch_fused(const LayerParams& p, const FusedPlan& plan, uint32_t fu
     return hipLaunchKernel(plan.kernel, dim3(plan.nwg), dim3(plan.threads), args, plan.smem, s);
 }
 
+
+// ------------------------------------------------------------------------------------ probe
+namespace {
+template <int TILE>
+__global__ __launch_bounds__(512, 1) void mfma_probe_kernel(const uint32_t* data, float* sink, uint32_t iterations) {
+    // eight operand fragments of each kind per lane, as a 128 x 64 wavefront tile keeps them around
+    bf16x8 fa[8], fb[8];
+    const u32x4* pool = reinterpret_cast<const u32x4*>(data);
+    constexpr uint32_t kMask = uint32_t(kMfmaProbeWords / 4 - 1);
+#pragma unroll
+    for (uint32_t i = 0; i < 8; ++i) {
+        fa[i] = __builtin_bit_cast(bf16x8, pool[(blockIdx.x * 512u + threadIdx.x + i * 4096u) & kMask]);
+        fb[i] = __builtin_bit_cast(bf16x8, pool[(blockIdx.x * 512u + threadIdx.x + i * 4096u + 77777u) & kMask]);
+    }
+    float total = 0.f;
+    if constexpr (TILE == 32) {
+        f32x16 acc[2][4] = {};
+        for (uint32_t it = 0; it < iterations; ++it)
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+                for (int n = 0; n < 2; ++n)
+#pragma unroll
+                    for (int m = 0; m < 4; ++m)
+                        acc[n][m] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[(n + 2 * ks) & 7], fa[(m + ks) & 7], acc[n][m], 0, 0, 0);
+        for (int n = 0; n < 2; ++n) for (int m = 0; m < 4; ++m) for (int i = 0; i < 16; ++i) total += acc[n][m][i];
+    } else {
+        f32x4 acc[4][8] = {};
+        for (uint32_t it = 0; it < iterations; ++it)
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+                for (int n = 0; n < 4; ++n)
+#pragma unroll
+                    for (int m = 0; m < 8; ++m)
+                        acc[n][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fb[(n + 4 * ks) & 7], fa[(m + ks) & 7], acc[n][m], 0, 0, 0);
+        for (int n = 0; n < 4; ++n) for (int m = 0; m < 8; ++m) for (int i = 0; i < 4; ++i) total += acc[n][m][i];
+    }
+    if (total == 12345.678f) *sink = total;   // keeps the loop alive; never true in practice
+}
+
+__global__ void mfma_probe_fill_kernel(uint32_t* data, size_t words, uint32_t zero) {
+    for (size_t i = size_t(blockIdx.x) * blockDim.x + threadIdx.x; i < words; i += size_t(gridDim.x) * blockDim.x) {
+        uint32_t h = uint32_t(i) * 2654435761u + 12345u;
+        h ^= h >> 15; h *= 2246822519u; h ^= h >> 13; h *= 3266489917u; h ^= h >> 16;
+        // two bf16: sign and 7 mantissa bits random, exponent 0x7e or 0x7f (0.5 <= |v| < 2)
+        const uint32_t lo = (h & 0x80ffu) | 0x3f00u, hi = ((h >> 16) & 0x80ffu) | 0x3f00u;
+        data[i] = zero ? 0u : (lo | (hi << 16));
+    }
+}
+}  // namespace
+
+hipError_t launch_mfma_probe(int tile, uint32_t iterations, const uint32_t* data, float* sink, int num_cus, double* flop,
+                             hipStream_t s) {
+    if (tile != 16 && tile != 32) return hipErrorInvalidValue;
+    // per iteration and wavefront: a 128 x 64 tile advanced by 64 values of K
+    if (flop) *flop = double(num_cus) * 8.0 * double(iterations) * 2.0 * 128.0 * 64.0 * 64.0;
+    if (tile == 32) hipLaunchKernelGGL(mfma_probe_kernel<32>, dim3(num_cus), dim3(512), 0, s, data, sink, iterations);
+    else hipLaunchKernelGGL(mfma_probe_kernel<16>, dim3(num_cus), dim3(512), 0, s, data, sink, iterations);
+    return hipGetLastError();
+}
+
+hipError_t launch_mfma_probe_fill(uint32_t* data, size_t words, bool zero, hipStream_t s) {
+    hipLaunchKernelGGL(mfma_probe_fill_kernel, dim3(2048), dim3(256), 0, s, data, words, zero ? 1u : 0u);
+    return hipGetLastError();
+}
+
 }  // namespace kleos_amd

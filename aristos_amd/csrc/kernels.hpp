@@ -37,6 +37,18 @@ hipError_t plan_fused(const LayerParams& p, int dtype, int num_cus, FusedPlan* p
 // schedule: a KLEOS_SCHEDULE_* value.
 hipError_t launch_fused(const LayerParams& p, const FusedPlan& plan, uint32_t fused_seq, int schedule, hipStream_t s);
 
+// Measurement probe, no part of the layer: one launch of a loop of bf16 matrix instructions on
+// operands held in registers (no LDS, no memory traffic inside the loop), on every CU, eight
+// wavefronts each. tile 32: 32x32x16 instructions, tile 16: 16x16x32. `data`: at least
+// kMfmaProbeWords 32-bit words the operands are drawn from (their bit patterns decide what the
+// multipliers toggle), `sink`: one float nobody reads. Returns the flop count of the launch in *flop.
+constexpr size_t kMfmaProbeWords = size_t(1) << 22;
+hipError_t launch_mfma_probe(int tile, uint32_t iterations, const uint32_t* data, float* sink, int num_cus, double* flop,
+                             hipStream_t s);
+// Fills `words` 32-bit words with pairs of bf16 values of random sign and mantissa and exponents close to 1
+// (zero = true: with zeros).
+hipError_t launch_mfma_probe_fill(uint32_t* data, size_t words, bool zero, hipStream_t s);
+
 // Why a configuration cannot run, or nullptr when it can.
 const char* unsupported_reason(uint32_t E, uint32_t k);
 

@@ -72,6 +72,15 @@ def set_mode(mode: int) -> None:
     _capi.check(_capi.lib().kleos_set_mode(int(mode)))
 
 
+def debug_mfma_probe(tile: int, iterations: int = 20000, zero_operands: bool = False) -> dict:
+    """One launch of the matrix-instruction probe (tile 32: 32x32x16 bf16 instructions, tile 16:
+    16x16x32) on every CU: its duration and the rate it ran at. Needs no initialised context."""
+    ms = C.c_float(0.0)
+    flop = C.c_double(0.0)
+    _capi.check(_capi.lib().kleos_debug_mfma_probe(int(tile), int(iterations), int(bool(zero_operands)), C.byref(ms), C.byref(flop)))
+    return {"ms": float(ms.value), "tflops": float(flop.value) / (float(ms.value) * 1e-3) / 1e12}
+
+
 def set_schedule(schedule: int) -> None:
     """SCHEDULE_AUTO (default), SCHEDULE_DYNAMIC or SCHEDULE_STATIC: how the persistent launch hands
     out expert tiles."""

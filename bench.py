@@ -1,7 +1,7 @@
 """Benchmark of the fused MoE-layer forward on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu-baseline]
-                    [--power-seconds S] [--zero-expert-weights] [--calib-gemm M,N,K]
+                    [--power-seconds S] [--zero-expert-weights] [--calib-gemm M,N,K] [--calib-mfma]
 
 A step is one forward of the layer (one persistent kernel launch) over one batch of synthetic
 tokens already resident in HBM. The per-phase figures are measured first, with launch counts of
@@ -157,6 +157,24 @@ def vendor_gemm_calibration(shape: str, seconds: float, zero_a: bool) -> int:
     return 0
 
 
+def mfma_calibration(seconds: float, zero: bool) -> int:
+    """`--calib-mfma`: the library's matrix-instruction probe (bf16 operands held in registers, no
+    memory traffic) looped for `seconds` per instruction: what the matrix cores sustain, at which
+    socket power, with 32x32x16 and with 16x16x32 instructions. One JSON line per instruction."""
+    import aristos_amd as ka
+    for tile in (32, 16, 32, 16):
+        rates = []
+        power = sustained_power(max(3.0, seconds), lambda: rates.append(ka.moe.debug_mfma_probe(tile, 20000, zero)["tflops"]))
+        tail = rates[len(rates) // 2:]
+        tf = sum(tail) / len(tail)
+        print(json.dumps({"calibration": "bf16 matrix instructions on register operands, all CUs",
+                          "instruction": "v_mfma_f32_32x32x16_bf16" if tile == 32 else "v_mfma_f32_16x16x32_bf16",
+                          "operands": "zeros" if zero else "random values of unit size", "tflops": round(tf, 1),
+                          "mfma_frac": round(tf / PEAK_BF16_TFLOPS, 4), "power": power,
+                          "joule_per_tflop": round(power["mean_w"] / tf, 4) if power else None}))
+    return 0
+
+
 PHASED_SKIP, FUSED_SKIP, REHEARSALS = 8, 32, 3
 
 
@@ -199,6 +217,9 @@ def main() -> int:
                     help="M,N,K: instead of the layer, loop the vendor's bf16 GEMM of that shape for "
                          "--power-seconds and report its TFLOP/s and socket power (add --zero-expert-weights "
                          "to zero its first operand)")
+    ap.add_argument("--calib-mfma", action="store_true",
+                    help="instead of the layer, loop the library's matrix-instruction probe for --power-seconds per "
+                         "instruction and report TFLOP/s and socket power (--zero-expert-weights: zero operands)")
     ap.add_argument("--print-fingerprint", action="store_true",
                     help="print the fingerprint of the library sources (recorded in the counter summaries) and exit")
     args = ap.parse_args()
@@ -223,6 +244,8 @@ def main() -> int:
     torch.cuda.set_device(0)
     if args.calib_gemm:
         return vendor_gemm_calibration(args.calib_gemm, args.power_seconds, args.zero_expert_weights)
+    if args.calib_mfma:
+        return mfma_calibration(args.power_seconds, args.zero_expert_weights)
     w = synth.WORKLOADS[args.workload]
     iP, d = synth.make_inputs(w, seed=args.seed, device="cuda")
     if args.zero_expert_weights:

@@ -322,6 +322,15 @@ int kleos_debug_static_scratch_expiry(unsigned long long ticks, uint32_t skip_la
  * kleos_last_error(). Touches no device: lets a test pin, for instance, what a refused cooperative
  * launch (hipErrorCooperativeLaunchTooLarge) looks like to a caller. */
 int kleos_debug_map_hip_error(int hip_error);
+/* Measurement probe with no counterpart in the reference and no part in the layer: one launch, on the
+ * current device's null stream, of a loop of bf16 matrix instructions on operands held in registers
+ * (eight wavefronts on every CU, no LDS or memory traffic inside the loop), timed by events. tile 32
+ * issues 32x32x16 instructions, tile 16 issues 16x16x32; operands are random bf16 values of unit size,
+ * or zeros. *ms: duration of the launch, *flop: its floating-point operations. What the matrix cores
+ * sustain at the package's power cap, and how that depends on the instruction and on the data, is
+ * what bounds the expert GEMM (bench.py --calib-mfma samples the socket power around it). Keeps
+ * 16 MB of device memory until the process ends. */
+int kleos_debug_mfma_probe(int tile, uint32_t iterations, int zero_operands, float* ms, double* flop);
 
 /* ---- errors --------------------------------------------------------------------------------- */
 /* Replaces the KLEOS_CHECK_CUDA / KLEOS_ASSERT message conventions (csrc/include/kleos/debug.cuh:

@@ -490,6 +490,19 @@ def test_timing_interfaces_of_the_persistent_launch():
     assert st["foreign_tiles"] <= st["tiles"]
 
 
+def test_matrix_instruction_probe_runs_and_reports_a_rate():
+    """kleos_debug_mfma_probe: both instructions, random and zero operands, give a positive duration
+    and a rate below the published peak; bad arguments are refused."""
+    for tile in (32, 16):
+        for zero in (False, True):
+            r = ka.moe.debug_mfma_probe(tile, iterations=2000, zero_operands=zero)
+            assert r["ms"] > 0 and 100.0 < r["tflops"] < 2600.0, (tile, zero, r)
+    with pytest.raises(ka.KleosError):
+        ka.moe.debug_mfma_probe(8, 100)
+    with pytest.raises(ka.KleosError):
+        ka.moe.debug_mfma_probe(16, 0)
+
+
 def test_cooperative_launch_gives_the_same_bits():
     """kleos_set_cooperative_launch(1): the runtime checks the grid's residency at every launch; the
     kernel and its results are the same."""
