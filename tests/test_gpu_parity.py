@@ -413,6 +413,48 @@ def test_experts_that_fill_a_tile_to_every_quarter(mode):
     assert (v["topk_slot"] < 0).sum() > 0
 
 
+def _one_hot_layer(c, rows, seed):
+    """A layer whose token t goes to one chosen expert (k = 1): `rows[e]` tokens to expert e, the rest to
+    the last expert; one-hot input features that the gate weights pick up decide it."""
+    x, wg, w_up, w_down, b_up, b_down = random_layer(c, seed=seed, w_std=0.08, bias_std=0.1)
+    E = c.E
+    first = np.repeat(np.arange(E), rows)
+    assert first.size == c.S
+    np.random.default_rng(seed).shuffle(first)
+    x[:, :E] = 0.0
+    x[np.arange(c.S), first] = 8.0
+    wg[:, :E] = np.eye(E, dtype=np.float32)
+    wg[:, E:] *= 0.25
+    return pack_inputs(c, x, wg, w_up, w_down, b_up, b_down)
+
+
+@pytest.mark.parametrize("mode", MODES, ids=MODE_IDS)
+@pytest.mark.parametrize("variant", ["256-row tiles", "128-row tiles"])
+def test_experts_that_end_inside_and_at_the_edges_of_16_row_blocks(mode, variant):
+    """A wavefront computes only the blocks of 16 rows that hold rows of its tile (four versions of the
+    main loop, for 1 to 4 blocks of its 64 rows). Experts of 1, 15, 16, 17, 31, 33, 47, 48, 49, 63, 64, 65,
+    ... rows put the last row at the start, inside and at the end of every such block, in the 256-row
+    tile (capacity 256) and in the 128-row tile (capacity 128)."""
+    if variant == "256-row tiles":
+        rows = [1, 15, 16, 17, 31, 33, 47, 48, 49, 63, 64, 65, 100, 129, 200, 255]
+        S, E = 2048, 32
+        rows = rows + [17] * 15
+        rows.append(S - sum(rows))                   # the last expert takes the rest (and overflows its capacity)
+        keys = _keys(S, 128, 256, E, 1, cf=4.0)      # EC = 256
+    else:
+        rows = [1, 15, 16, 17, 31, 33, 47, 48, 49, 63, 64, 65, 79, 81, 100, 127]
+        S, E = 1024, 32
+        rows = rows + [9] * 15
+        rows.append(S - sum(rows))
+        keys = _keys(S, 128, 256, E, 1, cf=4.0)      # EC = 128
+    c = moe_ref.cfg_from_keys(keys)
+    assert c.EC == (256 if variant == "256-row tiles" else 128)
+    iP = _one_hot_layer(c, rows, seed=97)
+    d, v, moe_out, err = check_against_oracle(c, keys, iP, mode)
+    np.testing.assert_array_equal(v["expert_count"], np.array(rows))
+    assert (v["topk_slot"] < 0).sum() == max(0, rows[-1] - c.EC)      # only the last expert can drop tokens
+
+
 @pytest.mark.parametrize("mode", MODES, ids=MODE_IDS)
 def test_back_to_back_launches_need_no_host_reset(mode):
     """The reference resets its state inside the kernel (moe.cuh:31-70) so launches can follow each
