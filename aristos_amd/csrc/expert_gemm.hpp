@@ -20,10 +20,11 @@ namespace kleos_amd {
 // of the instruction land in 1 KB of consecutive LDS). They never occupy a vector register. Rows of
 // A are gathered through the slot->token table by giving each lane its token's row address.
 // Slice kt+STAGES-1 is requested during slice kt, into the stage slice kt-1 was read from, its loads
-// placed one by one behind the matrix instructions of the slice's first K steps.
+// placed one by one behind the matrix instructions of the slice's first quarters (a slice's matrix
+// instructions run in four equal quarters: one K step each with 32x32x16, half a K step with 16x16x32).
 // With two stages the loads can instead run two slices ahead (AHEAD2): slice kt+2 is requested
 // into the stage of slice kt as soon as every wavefront has read its last fragments of slice kt (a
-// second workgroup barrier per slice, placed before the last K step, whose matrix instructions
+// second workgroup barrier per slice, placed before the last quarter, whose matrix instructions
 // the loads then follow one by one), so the memory pipeline holds requests across the wait for
 // slice kt+1 instead of running empty at every slice boundary.
 //
@@ -47,7 +48,6 @@ namespace kleos_amd {
 // keeps turning across tiles (finish() stages its output in the stage of the last slice, which
 // every wavefront has left; begin() follows behind a workgroup barrier of the caller).
 // ------------------------------------------------------------------------------------------------
-typedef const __attribute__((address_space(1))) void* global_cptr;
 typedef __attribute__((address_space(3))) void* lds_ptr;
 
 // One direct global->LDS load: every lane names 16 bytes of global memory, and the 64 lanes' bytes
@@ -260,8 +260,8 @@ __device__ __forceinline__ void static_for(F&& f) {
 // dominates it needs SPREAD to pay (8-expert shape with hidden size 4096, both projections: 4.18 ms
 // with all loads of a slice at once against 4.11 one slice ahead, 3.95 with them shared out 4 + 4).
 // SPREAD (with AHEAD2): when the loads of a slice are issued. 0: all of them behind the matrix
-// instructions of the last K step of the slice two before it, which frees their stage. Otherwise
-// only the first of them go there and the rest behind the first K steps of the next slice
+// instructions of the last quarter of the slice two before it, which frees their stage. Otherwise
+// only the first of them go there and the rest behind the first quarters of the next slice
 // (spread_count: 1 = 4 + 4, 2 = 3 + 3 + 2 of the 8 loads of a wavefront). The CU's load path takes in
 // about one 1 KB load every 36 clocks while all CUs stream; the 64 loads of a slice issued by eight
 // wavefronts inside one K step queue up in front of it, and each wavefront's matrix instructions sit
@@ -305,8 +305,8 @@ struct Gemm16 {
     static constexpr int kQuarters = 4;                            // a slice's matrix instructions in four equal runs
     static constexpr int kPerQuarter = TN * TM * kSteps / kQuarters;
     static constexpr int kPanelRows = kEpiloguePanelRows;          // epilogue staging: 32 rows x 64 columns per wavefront
-    // loads of a slice (per wavefront) issued at the last K step of the slice two before it [0] and at
-    // K steps 0, 1, 2 of the slice before it [1..3]
+    // loads of a slice (per wavefront) issued at the last quarter of the slice two before it [0] and at
+    // quarters 0, 1, 2 of the slice before it [1..3]
     static constexpr int spread_count(int i) {
         constexpr int L = LA + LB;
         switch (SPREAD) {
@@ -613,11 +613,11 @@ struct Gemm16 {
             constexpr int N0 = spread_count(0), N1 = spread_count(1), N2 = spread_count(2), N3 = spread_count(3);
             // Slice 0 was requested by begin(). Every wavefront has left the previous tile's epilogue,
             // which staged its output in the stage slice 1 goes to: its first loads go out here, the
-            // others behind the first K steps of slice 0.
+            // others behind the first quarters of slice 0.
             asm volatile("s_barrier" ::: "memory");
             if (t.k_tiles > 1) issue_range<0, N0>(t, smem, 1);
-            // One slice: `next_tag` - slice kt+1 exists (its loads N0 .. are issued behind K steps 0 to 2),
-            // `next2_tag` - slice kt+2 exists (its first N0 loads go behind the last K step, into the
+            // One slice: `next_tag` - slice kt+1 exists (its loads N0 .. are issued behind quarters 0 to 2),
+            // `next2_tag` - slice kt+2 exists (its first N0 loads go behind the last quarter, into the
             // stage of slice kt, once every wavefront has read its last fragments of it).
             auto slice = [&](uint32_t kt, auto next_tag, auto next2_tag) {
                 constexpr bool NEXT = decltype(next_tag)::value, NEXT2 = decltype(next2_tag)::value;

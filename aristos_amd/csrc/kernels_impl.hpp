@@ -54,8 +54,9 @@ constexpr int kXcds = 8;
 // weight tile is shared by several workgroups through L2, loads return quickly and the matrix work
 // dominates): the tile of variant 0 on 2 x 4 wavefronts of 128 x 64 (3.53 against 3.57 ms with 4 x 2
 // at the 8-expert shape with hidden size 4096), the loads two slices ahead like variant 0 and shared
-// out 4 + 4 over two K steps (both projections of that shape on random data: 3.95 ms against 4.11 with
-// the loads one slice ahead, all behind the first K step, and 4.18 two slices ahead all at once).
+// out 4 + 4 over two quarters of a slice (both projections of that shape on random data, 32x32x16
+// instructions: 3.95 ms against 4.11 with the loads one slice ahead, all behind the first K step, and 4.18
+// two slices ahead all at once).
 // Variants 0 and 1 load their weight rows non-temporally (headline 378 against 390 us per forward,
 // the 16-expert shape 192 against 196, the 256-expert shape 3.43 against 3.48 ms); variant 2, whose
 // weight tiles are shared by eight workgroups and more, does not (4.06 against 4.01 ms with it).
@@ -64,7 +65,7 @@ constexpr int kXcds = 8;
 #define KLEOS_TUNE_V0_SPREAD 1       // variant 0: loads of a slice issued 4 + 4 over two quarters of a slice (2: 3 + 3 + 2)
 #endif
 #ifndef KLEOS_TUNE_V2_SPREAD
-#define KLEOS_TUNE_V2_SPREAD 1       // variant 2: two slices ahead, 4 + 4 over two K steps; -1: one slice ahead
+#define KLEOS_TUNE_V2_SPREAD 1       // variant 2: two slices ahead, 4 + 4 over two quarters of a slice; -1: one slice ahead
 #endif
 #ifndef KLEOS_TUNE_ZERO_PAD
 #define KLEOS_TUNE_ZERO_PAD 1      // activation rows past an expert's last row read zeros instead of its last row
