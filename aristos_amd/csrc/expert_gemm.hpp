@@ -312,19 +312,10 @@ struct Gemm16 {
         switch (SPREAD) {
             case 1: return i < 2 ? L / 2 : 0;                                                       // 4 4 0 0
             case 2: return i == 0 || i == 1 ? (3 * L) / 8 : (i == 2 ? L - 2 * ((3 * L) / 8) : 0);   // 3 3 2 0
-#ifdef KLEOS_X_SPREADS
-            case 3: return L / 4;                                                                   // 2 2 2 2
-            case 4: return i == 0 ? L / 4 : (i == 1 ? (3 * L) / 4 : 0);                             // 2 6 0 0
-            case 5: return i == 0 ? (3 * L) / 4 : (i == 1 ? L / 4 : 0);                             // 6 2 0 0
-            case 6: return i == 0 ? L / 2 : (i == 1 || i == 2 ? L / 4 : 0);                         // 4 2 2 0
-            case 7: return i == 1 ? L / 2 : (i == 0 || i == 2 ? L / 4 : 0);                         // 2 4 2 0
-#endif
             default: return i == 0 ? L : 0;                                                         // all at once
         }
     }
-#ifndef KLEOS_X_SPREADS
     static_assert(SPREAD >= 0 && SPREAD <= 2);
-#endif
     static_assert(SPREAD == 0 || (AHEAD2 && (LA + LB) % 8 == 0));
     static_assert(spread_count(0) + spread_count(1) + spread_count(2) + spread_count(3) == LA + LB);
     static_assert(BK == 32 || BK == 64);
@@ -521,171 +512,171 @@ struct Gemm16 {
         // them are left out of the fragment reads and the matrix instructions (with the 16-row tiles, in
         // the configurations that take the trouble: kBlockSkip); their accumulators are never stored.
         auto body = [&](auto xb_tag) {
-        constexpr int XB = decltype(xb_tag)::value;
-        auto x_block_used = [](int mi) { return mi < XB; };
-        vec8 fw[2][MI == 32 ? TN : 1], fx[2][MI == 32 ? TM : 1];
-        vec8 fo[MI == 16 ? NO : 1], fi[2][MI == 16 ? NI : 1];
-        const int base_o = kOuterX ? base_x : base_w, base_i = kOuterX ? base_w : base_x;
-        auto read_fragments = [&](const char* st, int ks) {
-            if constexpr (MI == 32) {
-#pragma unroll
-                for (int ni = 0; ni < TN; ++ni) fw[ks & 1][ni] = __builtin_bit_cast(vec8, load16(st + (base_w ^ (ks << kStepShift)) + ni * MI * kRowBytes));
-#pragma unroll
-                for (int mi = 0; mi < TM; ++mi) fx[ks & 1][mi] = __builtin_bit_cast(vec8, load16(st + (base_x ^ (ks << kStepShift)) + mi * MI * kRowBytes));
-            } else {
-#pragma unroll
-                for (int k = 0; k < NI; ++k)
-                    if (kOuterX || x_block_used(k)) fi[ks & 1][k] = __builtin_bit_cast(vec8, load16(st + (base_i ^ (ks << kStepShift)) + k * MI * kRowBytes));
-#pragma unroll
-                for (int o = 0; o < NO; ++o)
-                    if (!kOuterX || x_block_used(o)) fo[o] = __builtin_bit_cast(vec8, load16(st + (base_o ^ (ks << kStepShift)) + o * MI * kRowBytes));
-            }
-        };
-        // Where one load of slice kn comes from and goes to (load li < LA: activation rows, else weight rows).
-        struct SliceLoads { uint32_t sa, sb, k0; };
-        const uint32_t lds_wave = lds_address(smem) + 1024 * wave_index();
-        auto loads_of = [&](uint32_t kn) {
-            SliceLoads l;
-            l.sa = lds_wave + stage_of(t, kn) * kStage;
-            l.sb = l.sa + kABytes;
-            uint32_t slice = kn + t.k_first;
-            slice = slice >= t.k_tiles ? slice - t.k_tiles : slice;
-            l.k0 = slice * BK;
-            return l;
-        };
-        // A quarter of a slice's matrix instructions (one K step with the 32-row tiles, half a K step
-        // with the 16-row tiles) in a pinned order: one matrix instruction, behind it one LDS read of the
-        // next K step's fragments (behind the first TN + TM instructions of a step) and, with LOADS, one
-        // global load of a later slice, and again. Issued as blocks - all reads, then all
-        // matrix instructions - the two wavefronts of a SIMD took turns instead of overlapping, and a
-        // slice's loads in a block in front of a K step held the matrix cores up (8 experts x 2560
-        // rows, hidden size 4096, both projections: 3.80 ms in blocks, 3.49 with the reads interleaved,
-        // 3.47 with the loads interleaved too; with operands resident in L2 3.49, 2.96 and 2.72).
-        // The loads are a compile-time switch: a branch around matrix instructions makes the compiler keep
-        // two copies of the accumulators.
-        // `first_tag`, `count_tag`: the quarter carries the loads first .. first + count - 1 of the slice `l`
-        // describes, evenly spaced behind its matrix instructions (count 0: none).
-        auto quarter = [&](const char* st, auto q_tag, const SliceLoads& l, auto first_tag, auto count_tag) {
-            constexpr int Q = decltype(q_tag)::value, FIRST = decltype(first_tag)::value, COUNT = decltype(count_tag)::value;
-            constexpr int kParts = kQuarters / kSteps;                 // quarters per K step
-            constexpr int ks = Q / kParts, part = Q % kParts;
-            static_assert(COUNT <= kPerQuarter);
-            constexpr int kEvery = kPerQuarter / (COUNT > 0 ? COUNT : 1);
-#pragma unroll
-            for (int j = 0; j < kPerQuarter; ++j) {
-                __builtin_amdgcn_sched_barrier(0);
-                const int i = part * kPerQuarter + j;                  // the step's i-th matrix instruction
+            constexpr int XB = decltype(xb_tag)::value;
+            auto x_block_used = [](int mi) { return mi < XB; };
+            vec8 fw[2][MI == 32 ? TN : 1], fx[2][MI == 32 ? TM : 1];
+            vec8 fo[MI == 16 ? NO : 1], fi[2][MI == 16 ? NI : 1];
+            const int base_o = kOuterX ? base_x : base_w, base_i = kOuterX ? base_w : base_x;
+            auto read_fragments = [&](const char* st, int ks) {
                 if constexpr (MI == 32) {
-                    const int ni = i / TM, mi = i % TM;
-                    acc[ni][mi] = Elem16<E>::mfma32(fw[ks & 1][ni], fx[ks & 1][mi], acc[ni][mi]);
-                    if (ks + 1 < kSteps) {
-                        const int nb = (ks + 1) & 1;
-                        if (i < TN) fw[nb][i] = __builtin_bit_cast(vec8, load16(st + (base_w ^ ((ks + 1) << kStepShift)) + i * MI * kRowBytes));
-                        else if (i < TN + TM) fx[nb][i - TN] = __builtin_bit_cast(vec8, load16(st + (base_x ^ ((ks + 1) << kStepShift)) + (i - TN) * MI * kRowBytes));
-                    }
+#pragma unroll
+                    for (int ni = 0; ni < TN; ++ni) fw[ks & 1][ni] = __builtin_bit_cast(vec8, load16(st + (base_w ^ (ks << kStepShift)) + ni * MI * kRowBytes));
+#pragma unroll
+                    for (int mi = 0; mi < TM; ++mi) fx[ks & 1][mi] = __builtin_bit_cast(vec8, load16(st + (base_x ^ (ks << kStepShift)) + mi * MI * kRowBytes));
                 } else {
-                    const int o = i / NI, k = i % NI;
-                    if (x_block_used(kOuterX ? o : k)) {   // (folds at compile time: o and k are unrolled)
-                        if constexpr (kOuterX) acc[k][o] = Elem16<E>::mfma16(fi[ks & 1][k], fo[o], acc[k][o]);
-                        else acc[o][k] = Elem16<E>::mfma16(fo[o], fi[ks & 1][k], acc[o][k]);
-                    }
-                    if (ks + 1 < kSteps) {
-                        // behind the last instruction that uses fo[o]: its successor; behind the first
-                        // instructions of the first NI outer rounds: the inner set of the next step
-                        if (k == NI - 1) {
-                            if (!kOuterX || x_block_used(o)) fo[o] = __builtin_bit_cast(vec8, load16(st + (base_o ^ ((ks + 1) << kStepShift)) + o * MI * kRowBytes));
-                        } else if (k == 0 && o < NI) {
-                            if (kOuterX || x_block_used(o)) fi[(ks + 1) & 1][o] = __builtin_bit_cast(vec8, load16(st + (base_i ^ ((ks + 1) << kStepShift)) + o * MI * kRowBytes));
+#pragma unroll
+                    for (int k = 0; k < NI; ++k)
+                        if (kOuterX || x_block_used(k)) fi[ks & 1][k] = __builtin_bit_cast(vec8, load16(st + (base_i ^ (ks << kStepShift)) + k * MI * kRowBytes));
+#pragma unroll
+                    for (int o = 0; o < NO; ++o)
+                        if (!kOuterX || x_block_used(o)) fo[o] = __builtin_bit_cast(vec8, load16(st + (base_o ^ (ks << kStepShift)) + o * MI * kRowBytes));
+                }
+            };
+            // Where one load of slice kn comes from and goes to (load li < LA: activation rows, else weight rows).
+            struct SliceLoads { uint32_t sa, sb, k0; };
+            const uint32_t lds_wave = lds_address(smem) + 1024 * wave_index();
+            auto loads_of = [&](uint32_t kn) {
+                SliceLoads l;
+                l.sa = lds_wave + stage_of(t, kn) * kStage;
+                l.sb = l.sa + kABytes;
+                uint32_t slice = kn + t.k_first;
+                slice = slice >= t.k_tiles ? slice - t.k_tiles : slice;
+                l.k0 = slice * BK;
+                return l;
+            };
+            // A quarter of a slice's matrix instructions (one K step with the 32-row tiles, half a K step
+            // with the 16-row tiles) in a pinned order: one matrix instruction, behind it one LDS read of the
+            // next K step's fragments (behind the first TN + TM instructions of a step) and, with LOADS, one
+            // global load of a later slice, and again. Issued as blocks - all reads, then all
+            // matrix instructions - the two wavefronts of a SIMD took turns instead of overlapping, and a
+            // slice's loads in a block in front of a K step held the matrix cores up (8 experts x 2560
+            // rows, hidden size 4096, both projections: 3.80 ms in blocks, 3.49 with the reads interleaved,
+            // 3.47 with the loads interleaved too; with operands resident in L2 3.49, 2.96 and 2.72).
+            // The loads are a compile-time switch: a branch around matrix instructions makes the compiler keep
+            // two copies of the accumulators.
+            // `first_tag`, `count_tag`: the quarter carries the loads first .. first + count - 1 of the slice `l`
+            // describes, evenly spaced behind its matrix instructions (count 0: none).
+            auto quarter = [&](const char* st, auto q_tag, const SliceLoads& l, auto first_tag, auto count_tag) {
+                constexpr int Q = decltype(q_tag)::value, FIRST = decltype(first_tag)::value, COUNT = decltype(count_tag)::value;
+                constexpr int kParts = kQuarters / kSteps;                 // quarters per K step
+                constexpr int ks = Q / kParts, part = Q % kParts;
+                static_assert(COUNT <= kPerQuarter);
+                constexpr int kEvery = kPerQuarter / (COUNT > 0 ? COUNT : 1);
+#pragma unroll
+                for (int j = 0; j < kPerQuarter; ++j) {
+                    __builtin_amdgcn_sched_barrier(0);
+                    const int i = part * kPerQuarter + j;                  // the step's i-th matrix instruction
+                    if constexpr (MI == 32) {
+                        const int ni = i / TM, mi = i % TM;
+                        acc[ni][mi] = Elem16<E>::mfma32(fw[ks & 1][ni], fx[ks & 1][mi], acc[ni][mi]);
+                        if (ks + 1 < kSteps) {
+                            const int nb = (ks + 1) & 1;
+                            if (i < TN) fw[nb][i] = __builtin_bit_cast(vec8, load16(st + (base_w ^ ((ks + 1) << kStepShift)) + i * MI * kRowBytes));
+                            else if (i < TN + TM) fx[nb][i - TN] = __builtin_bit_cast(vec8, load16(st + (base_x ^ ((ks + 1) << kStepShift)) + (i - TN) * MI * kRowBytes));
+                        }
+                    } else {
+                        const int o = i / NI, k = i % NI;
+                        if (x_block_used(kOuterX ? o : k)) {   // (folds at compile time: o and k are unrolled)
+                            if constexpr (kOuterX) acc[k][o] = Elem16<E>::mfma16(fi[ks & 1][k], fo[o], acc[k][o]);
+                            else acc[o][k] = Elem16<E>::mfma16(fo[o], fi[ks & 1][k], acc[o][k]);
+                        }
+                        if (ks + 1 < kSteps) {
+                            // behind the last instruction that uses fo[o]: its successor; behind the first
+                            // instructions of the first NI outer rounds: the inner set of the next step
+                            if (k == NI - 1) {
+                                if (!kOuterX || x_block_used(o)) fo[o] = __builtin_bit_cast(vec8, load16(st + (base_o ^ ((ks + 1) << kStepShift)) + o * MI * kRowBytes));
+                            } else if (k == 0 && o < NI) {
+                                if (kOuterX || x_block_used(o)) fi[(ks + 1) & 1][o] = __builtin_bit_cast(vec8, load16(st + (base_i ^ ((ks + 1) << kStepShift)) + o * MI * kRowBytes));
+                            }
                         }
                     }
+                    if constexpr (COUNT > 0) {
+                        if (j % kEvery == 0 && j / kEvery < COUNT) issue_one(t, l.sa, l.sb, l.k0, FIRST + j / kEvery);
+                    }
                 }
-                if constexpr (COUNT > 0) {
-                    if (j % kEvery == 0 && j / kEvery < COUNT) issue_one(t, l.sa, l.sb, l.k0, FIRST + j / kEvery);
-                }
-            }
-            __builtin_amdgcn_sched_barrier(0);
-        };
-        using Q0 = std::integral_constant<int, 0>; using Q1 = std::integral_constant<int, 1>;
-        using Q2 = std::integral_constant<int, 2>; using Q3 = std::integral_constant<int, 3>;
-        static_assert(MI == 16 || TN + TM <= kPerQuarter, "the first quarter of a K step has a matrix instruction for every fragment read");
-        if constexpr (AHEAD2) {
-            static_assert(LA + LB <= kPerQuarter, "the loads of a slice fit behind the matrix instructions of one quarter");
-            constexpr int N0 = spread_count(0), N1 = spread_count(1), N2 = spread_count(2), N3 = spread_count(3);
-            // Slice 0 was requested by begin(). Every wavefront has left the previous tile's epilogue,
-            // which staged its output in the stage slice 1 goes to: its first loads go out here, the
-            // others behind the first quarters of slice 0.
-            asm volatile("s_barrier" ::: "memory");
-            if (t.k_tiles > 1) issue_range<0, N0>(t, smem, 1);
-            // One slice: `next_tag` - slice kt+1 exists (its loads N0 .. are issued behind quarters 0 to 2),
-            // `next2_tag` - slice kt+2 exists (its first N0 loads go behind the last quarter, into the
-            // stage of slice kt, once every wavefront has read its last fragments of it).
-            auto slice = [&](uint32_t kt, auto next_tag, auto next2_tag) {
-                constexpr bool NEXT = decltype(next_tag)::value, NEXT2 = decltype(next2_tag)::value;
-                // this wavefront's loads of slice kt are complete once only the first N0 of slice kt+1
-                // are outstanding (the stores of the previous tile's epilogue are older than both)
-                if constexpr (NEXT) wait_vmcnt<N0>();
-                else wait_vmcnt<0>();
-                asm volatile("s_barrier" ::: "memory");   // every wavefront's share of slice kt is in LDS
-                if (kt == 0) after_first_barrier();
-                const char* st = smem + stage_of(t, kt) * kStage;
-                read_fragments(st, 0);
-                const SliceLoads l1 = NEXT ? loads_of(kt + 1) : SliceLoads{};
-                quarter(st, Q0{}, l1, std::integral_constant<int, N0>{}, std::integral_constant<int, NEXT ? N1 : 0>{});
-                quarter(st, Q1{}, l1, std::integral_constant<int, N0 + N1>{}, std::integral_constant<int, NEXT ? N2 : 0>{});
-                quarter(st, Q2{}, l1, std::integral_constant<int, N0 + N1 + N2>{}, std::integral_constant<int, NEXT ? N3 : 0>{});
-                if constexpr (NEXT2) {
-                    // this wavefront's last reads of the stage have returned; once that holds for every
-                    // wavefront the stage takes slice kt+2
-                    __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0)
-                    asm volatile("s_barrier" ::: "memory");
-                }
-                const SliceLoads l2 = NEXT2 ? loads_of(kt + 2) : SliceLoads{};
-                quarter(st, Q3{}, l2, std::integral_constant<int, 0>{}, std::integral_constant<int, NEXT2 ? N0 : 0>{});
+                __builtin_amdgcn_sched_barrier(0);
             };
-            const uint32_t ahead = t.k_tiles >= 2 ? t.k_tiles - 2 : 0u;   // slices that request slice kt+2
-            for (uint32_t kt = 0; kt < ahead; ++kt) slice(kt, std::true_type{}, std::true_type{});
-            if (t.k_tiles >= 2) slice(t.k_tiles - 2, std::true_type{}, std::false_type{});
-            slice(t.k_tiles - 1, std::false_type{}, std::false_type{});
-        } else {
-            static_assert(LA + LB <= kQuarters * kPerQuarter, "the loads of a slice fit behind the matrix instructions of a slice");
-            auto top = [&](uint32_t kt) {
-                // This wavefront's loads of slice kt are complete once only those of the later slices
-                // already issued (STAGES-2 of them, fewer at the end of the tile) are outstanding.
-                const uint32_t later = t.k_tiles - 1 - kt;
-                if (STAGES >= 4 && later >= 2) wait_vmcnt<(STAGES >= 4 ? 2 : 0) * kLoadsPerSlice>();
-                else if (STAGES >= 3 && later >= 1) wait_vmcnt<kLoadsPerSlice>();
-                else wait_vmcnt<0>();
-                // every wavefront's share of slice kt is in LDS, and everyone has finished with the stage
-                // the next loads overwrite (slice kt-1, or the previous tile's epilogue staging)
+            using Q0 = std::integral_constant<int, 0>; using Q1 = std::integral_constant<int, 1>;
+            using Q2 = std::integral_constant<int, 2>; using Q3 = std::integral_constant<int, 3>;
+            static_assert(MI == 16 || TN + TM <= kPerQuarter, "the first quarter of a K step has a matrix instruction for every fragment read");
+            if constexpr (AHEAD2) {
+                static_assert(LA + LB <= kPerQuarter, "the loads of a slice fit behind the matrix instructions of one quarter");
+                constexpr int N0 = spread_count(0), N1 = spread_count(1), N2 = spread_count(2), N3 = spread_count(3);
+                // Slice 0 was requested by begin(). Every wavefront has left the previous tile's epilogue,
+                // which staged its output in the stage slice 1 goes to: its first loads go out here, the
+                // others behind the first quarters of slice 0.
                 asm volatile("s_barrier" ::: "memory");
-                if (kt == 0) after_first_barrier();
-            };
-            // Quarter q carries the loads q * kPerQuarter ... of the slice STAGES-1 ahead, one behind each
-            // matrix instruction, until they run out (sharing them out evenly over the four K steps,
-            // which three stages would allow, changes nothing where it was measured: 2.93 against
-            // 2.92 ms per forward at the 256-expert top-8 shape, which is bound by HBM)
-            auto ksteps = [&](const char* st, const SliceLoads& l, auto loads_tag) {
-                static_for<kQuarters>([&](auto q_tag) {
-                    constexpr int q = decltype(q_tag)::value;
-                    constexpr int left = LA + LB - q * kPerQuarter;
-                    constexpr int count = !decltype(loads_tag)::value || left <= 0 ? 0 : (left < kPerQuarter ? left : kPerQuarter);
-                    quarter(st, q_tag, l, std::integral_constant<int, q * kPerQuarter>{}, std::integral_constant<int, count>{});
-                });
-            };
-            const uint32_t ahead = t.k_tiles >= uint32_t(STAGES - 1) ? t.k_tiles - (STAGES - 1) : 0u;   // slices that request a later one
-            for (uint32_t kt = 0; kt < ahead; ++kt) {
-                top(kt);
-                const char* st = smem + stage_of(t, kt) * kStage;
-                read_fragments(st, 0);
-                ksteps(st, loads_of(kt + STAGES - 1), std::true_type{});
+                if (t.k_tiles > 1) issue_range<0, N0>(t, smem, 1);
+                // One slice: `next_tag` - slice kt+1 exists (its loads N0 .. are issued behind quarters 0 to 2),
+                // `next2_tag` - slice kt+2 exists (its first N0 loads go behind the last quarter, into the
+                // stage of slice kt, once every wavefront has read its last fragments of it).
+                auto slice = [&](uint32_t kt, auto next_tag, auto next2_tag) {
+                    constexpr bool NEXT = decltype(next_tag)::value, NEXT2 = decltype(next2_tag)::value;
+                    // this wavefront's loads of slice kt are complete once only the first N0 of slice kt+1
+                    // are outstanding (the stores of the previous tile's epilogue are older than both)
+                    if constexpr (NEXT) wait_vmcnt<N0>();
+                    else wait_vmcnt<0>();
+                    asm volatile("s_barrier" ::: "memory");   // every wavefront's share of slice kt is in LDS
+                    if (kt == 0) after_first_barrier();
+                    const char* st = smem + stage_of(t, kt) * kStage;
+                    read_fragments(st, 0);
+                    const SliceLoads l1 = NEXT ? loads_of(kt + 1) : SliceLoads{};
+                    quarter(st, Q0{}, l1, std::integral_constant<int, N0>{}, std::integral_constant<int, NEXT ? N1 : 0>{});
+                    quarter(st, Q1{}, l1, std::integral_constant<int, N0 + N1>{}, std::integral_constant<int, NEXT ? N2 : 0>{});
+                    quarter(st, Q2{}, l1, std::integral_constant<int, N0 + N1 + N2>{}, std::integral_constant<int, NEXT ? N3 : 0>{});
+                    if constexpr (NEXT2) {
+                        // this wavefront's last reads of the stage have returned; once that holds for every
+                        // wavefront the stage takes slice kt+2
+                        __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0)
+                        asm volatile("s_barrier" ::: "memory");
+                    }
+                    const SliceLoads l2 = NEXT2 ? loads_of(kt + 2) : SliceLoads{};
+                    quarter(st, Q3{}, l2, std::integral_constant<int, 0>{}, std::integral_constant<int, NEXT2 ? N0 : 0>{});
+                };
+                const uint32_t ahead = t.k_tiles >= 2 ? t.k_tiles - 2 : 0u;   // slices that request slice kt+2
+                for (uint32_t kt = 0; kt < ahead; ++kt) slice(kt, std::true_type{}, std::true_type{});
+                if (t.k_tiles >= 2) slice(t.k_tiles - 2, std::true_type{}, std::false_type{});
+                slice(t.k_tiles - 1, std::false_type{}, std::false_type{});
+            } else {
+                static_assert(LA + LB <= kQuarters * kPerQuarter, "the loads of a slice fit behind the matrix instructions of a slice");
+                auto top = [&](uint32_t kt) {
+                    // This wavefront's loads of slice kt are complete once only those of the later slices
+                    // already issued (STAGES-2 of them, fewer at the end of the tile) are outstanding.
+                    const uint32_t later = t.k_tiles - 1 - kt;
+                    if (STAGES >= 4 && later >= 2) wait_vmcnt<(STAGES >= 4 ? 2 : 0) * kLoadsPerSlice>();
+                    else if (STAGES >= 3 && later >= 1) wait_vmcnt<kLoadsPerSlice>();
+                    else wait_vmcnt<0>();
+                    // every wavefront's share of slice kt is in LDS, and everyone has finished with the stage
+                    // the next loads overwrite (slice kt-1, or the previous tile's epilogue staging)
+                    asm volatile("s_barrier" ::: "memory");
+                    if (kt == 0) after_first_barrier();
+                };
+                // Quarter q carries the loads q * kPerQuarter ... of the slice STAGES-1 ahead, one behind each
+                // matrix instruction, until they run out (sharing them out evenly over the four K steps,
+                // which three stages would allow, changes nothing where it was measured: 2.93 against
+                // 2.92 ms per forward at the 256-expert top-8 shape, which is bound by HBM)
+                auto ksteps = [&](const char* st, const SliceLoads& l, auto loads_tag) {
+                    static_for<kQuarters>([&](auto q_tag) {
+                        constexpr int q = decltype(q_tag)::value;
+                        constexpr int left = LA + LB - q * kPerQuarter;
+                        constexpr int count = !decltype(loads_tag)::value || left <= 0 ? 0 : (left < kPerQuarter ? left : kPerQuarter);
+                        quarter(st, q_tag, l, std::integral_constant<int, q * kPerQuarter>{}, std::integral_constant<int, count>{});
+                    });
+                };
+                const uint32_t ahead = t.k_tiles >= uint32_t(STAGES - 1) ? t.k_tiles - (STAGES - 1) : 0u;   // slices that request a later one
+                for (uint32_t kt = 0; kt < ahead; ++kt) {
+                    top(kt);
+                    const char* st = smem + stage_of(t, kt) * kStage;
+                    read_fragments(st, 0);
+                    ksteps(st, loads_of(kt + STAGES - 1), std::true_type{});
+                }
+                for (uint32_t kt = ahead; kt < t.k_tiles; ++kt) {
+                    top(kt);
+                    const char* st = smem + stage_of(t, kt) * kStage;
+                    read_fragments(st, 0);
+                    ksteps(st, SliceLoads{}, std::false_type{});
+                }
             }
-            for (uint32_t kt = ahead; kt < t.k_tiles; ++kt) {
-                top(kt);
-                const char* st = smem + stage_of(t, kt) * kStage;
-                read_fragments(st, 0);
-                ksteps(st, SliceLoads{}, std::false_type{});
-            }
-        }
         };   // body
         if constexpr (kBlockSkip) {
             // (the same in all lanes of a wavefront; every version goes through the same barriers)
