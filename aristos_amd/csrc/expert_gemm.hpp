@@ -277,7 +277,20 @@ __device__ __forceinline__ void static_for(F&& f) {
 // writes half as many accumulator registers per multiply-add and draws less power for the same work
 // (instruction loops on random bf16 operands held in registers, whole device: 2.08 against 1.84
 // PFLOP/s at the same 1.31 kW), which is what bounds these kernels.
-template <typename E, int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES, bool STREAM_B, bool AHEAD2, int SPREAD = 0, int MI = 32>
+// RELEASE (with AHEAD2 and 16-row matrix tiles, whose slices have two K steps): where the barrier
+// that frees a slice's stage sits. The fragments of the second K step are read behind the matrix
+// instructions of the first, so a wavefront has finished with the stage half a slice before it
+// finishes the slice. 0: the barrier stays in front of the last quarter. 2: it moves into the third
+// quarter, kReleaseAt matrix instructions in (the last reads have returned by then), and the first
+// loads of the slice after the next follow it there: a quarter of a slice more for them to land
+// (8-expert shape with hidden size 4096: 3 088 against 3 115 us per forward; no difference at the
+// 64- and 16-expert shapes). 1: all loads of that slice go behind the early barrier, half in the third
+// and half in the last quarter, none into the next slice: every load has between one and one and a
+// half slices to land (16-expert shape 146 against 150 us, 64-expert shape 284 against 287 us; the
+// 8-expert shape loses, 3 177 against 3 115 us: its loads, bunched into half a slice, hold up the
+// matrix instructions behind them).
+template <typename E, int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES, bool STREAM_B, bool AHEAD2, int SPREAD = 0, int MI = 32,
+          int RELEASE = 0>
 struct Gemm16 {
     typedef typename Elem16<E>::vec8 vec8;
     typedef typename Elem16<E>::vec4 vec4;
@@ -302,6 +315,10 @@ struct Gemm16 {
     // rows that hold no rows of the tile (64-expert shape with skewed routing: the experts' 13 039 rows
     // take the matrix instructions of 13 424 rows that way, of 14 656 with whole wavefronts left out only)
     static constexpr bool kBlockSkip = KLEOS_GEMM_BLOCK_SKIP != 0 && MI == 16 && TM == 4;
+    static constexpr bool kEarlyRelease = RELEASE == 1;   // every load of a slice behind the early barrier of the slice two before it
+    static constexpr int kReleaseAt = 4;                  // matrix instructions of the third quarter in front of the early barrier
+    static_assert(RELEASE >= 0 && RELEASE <= 2);
+    static_assert(RELEASE == 0 || (AHEAD2 && MI == 16 && kSteps == 2));
     static constexpr int kQuarters = 4;                            // a slice's matrix instructions in four equal runs
     static constexpr int kPerQuarter = TN * TM * kSteps / kQuarters;
     static constexpr int kPanelRows = kEpiloguePanelRows;          // epilogue staging: 32 rows x 64 columns per wavefront
@@ -315,6 +332,8 @@ struct Gemm16 {
             default: return i == 0 ? L : 0;                                                         // all at once
         }
     }
+    static constexpr bool kEarlyFirst = RELEASE == 2;     // only the first loads move with the barrier; the others stay in the next slice
+    static_assert(RELEASE != 2 || spread_count(3) == 0, "the third quarter carries no loads of the next slice");
     static_assert(SPREAD >= 0 && SPREAD <= 2);
     static_assert(SPREAD == 0 || (AHEAD2 && (LA + LB) % 8 == 0));
     static_assert(spread_count(0) + spread_count(1) + spread_count(2) + spread_count(3) == LA + LB);
@@ -457,7 +476,21 @@ struct Gemm16 {
             // None of this wavefront's rows exist (an expert with few rows): it brings its share of
             // every slice into LDS at the same points of the same sequence of barriers as the others,
             // and leaves the fragment reads and the matrix instructions out.
-            if constexpr (AHEAD2) {
+            if constexpr (kEarlyRelease) {
+                constexpr int L = LA + LB;
+                asm volatile("s_barrier" ::: "memory");
+                if (t.k_tiles > 1) issue_range<0, L>(t, smem, 1);
+                for (uint32_t kt = 0; kt < t.k_tiles; ++kt) {
+                    if (kt + 1 < t.k_tiles) wait_vmcnt<L>();
+                    else wait_vmcnt<0>();
+                    asm volatile("s_barrier" ::: "memory");
+                    if (kt == 0) after_first_barrier();
+                    if (kt + 2 < t.k_tiles) {
+                        asm volatile("s_barrier" ::: "memory");
+                        issue_range<0, L>(t, smem, kt + 2);
+                    }
+                }
+            } else if constexpr (AHEAD2) {
                 constexpr int N0 = spread_count(0);
                 asm volatile("s_barrier" ::: "memory");
                 if (t.k_tiles > 1) issue_range<0, N0>(t, smem, 1);
@@ -556,15 +589,24 @@ struct Gemm16 {
             // two copies of the accumulators.
             // `first_tag`, `count_tag`: the quarter carries the loads first .. first + count - 1 of the slice `l`
             // describes, evenly spaced behind its matrix instructions (count 0: none).
-            auto quarter = [&](const char* st, auto q_tag, const SliceLoads& l, auto first_tag, auto count_tag) {
+            // `sync_tag` (S >= 0): in front of the quarter's S-th matrix instruction the wavefront waits for its LDS
+            // reads and for the workgroup; the quarter's loads come behind that point.
+            auto quarter = [&](const char* st, auto q_tag, const SliceLoads& l, auto first_tag, auto count_tag, auto sync_tag) {
                 constexpr int Q = decltype(q_tag)::value, FIRST = decltype(first_tag)::value, COUNT = decltype(count_tag)::value;
+                constexpr int S = decltype(sync_tag)::value, J0 = S > 0 ? S : 0;
                 constexpr int kParts = kQuarters / kSteps;                 // quarters per K step
                 constexpr int ks = Q / kParts, part = Q % kParts;
-                static_assert(COUNT <= kPerQuarter);
-                constexpr int kEvery = kPerQuarter / (COUNT > 0 ? COUNT : 1);
+                static_assert(COUNT <= kPerQuarter - J0);
+                constexpr int kEvery = (kPerQuarter - J0) / (COUNT > 0 ? COUNT : 1);
 #pragma unroll
                 for (int j = 0; j < kPerQuarter; ++j) {
                     __builtin_amdgcn_sched_barrier(0);
+                    if constexpr (S >= 0) {
+                        if (j == S) {
+                            __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0)
+                            asm volatile("s_barrier" ::: "memory");
+                        }
+                    }
                     const int i = part * kPerQuarter + j;                  // the step's i-th matrix instruction
                     if constexpr (MI == 32) {
                         const int ni = i / TM, mi = i % TM;
@@ -591,15 +633,45 @@ struct Gemm16 {
                         }
                     }
                     if constexpr (COUNT > 0) {
-                        if (j % kEvery == 0 && j / kEvery < COUNT) issue_one(t, l.sa, l.sb, l.k0, FIRST + j / kEvery);
+                        if (j >= J0 && (j - J0) % kEvery == 0 && (j - J0) / kEvery < COUNT) issue_one(t, l.sa, l.sb, l.k0, FIRST + (j - J0) / kEvery);
                     }
                 }
                 __builtin_amdgcn_sched_barrier(0);
             };
             using Q0 = std::integral_constant<int, 0>; using Q1 = std::integral_constant<int, 1>;
             using Q2 = std::integral_constant<int, 2>; using Q3 = std::integral_constant<int, 3>;
+            using NoSync = std::integral_constant<int, -1>;
             static_assert(MI == 16 || TN + TM <= kPerQuarter, "the first quarter of a K step has a matrix instruction for every fragment read");
-            if constexpr (AHEAD2) {
+            if constexpr (kEarlyRelease) {
+                // The barrier that frees the stage sits kReleaseAt matrix instructions into the second K step, and
+                // all loads of the slice after the next go out behind it, half in each quarter.
+                constexpr int L = LA + LB;
+                constexpr int AT = kReleaseAt;
+                constexpr int M2 = L / 2;
+                static_assert(M2 <= kPerQuarter - AT && L - M2 <= kPerQuarter);
+                using None = std::integral_constant<int, 0>;
+                asm volatile("s_barrier" ::: "memory");   // every wavefront has left the previous tile's epilogue, staged where slice 1 goes
+                if (t.k_tiles > 1) issue_range<0, L>(t, smem, 1);
+                auto slice = [&](uint32_t kt, auto next_tag, auto next2_tag) {
+                    constexpr bool NEXT = decltype(next_tag)::value, NEXT2 = decltype(next2_tag)::value;
+                    // this wavefront's loads of slice kt are complete once only those of slice kt+1 are outstanding
+                    if constexpr (NEXT) wait_vmcnt<L>();
+                    else wait_vmcnt<0>();
+                    asm volatile("s_barrier" ::: "memory");   // every wavefront's share of slice kt is in LDS
+                    if (kt == 0) after_first_barrier();
+                    const char* st = smem + stage_of(t, kt) * kStage;
+                    read_fragments(st, 0);
+                    quarter(st, Q0{}, SliceLoads{}, None{}, None{}, NoSync{});
+                    quarter(st, Q1{}, SliceLoads{}, None{}, None{}, NoSync{});
+                    const SliceLoads l2 = NEXT2 ? loads_of(kt + 2) : SliceLoads{};
+                    quarter(st, Q2{}, l2, None{}, std::integral_constant<int, NEXT2 ? M2 : 0>{}, std::integral_constant<int, NEXT2 ? AT : -1>{});
+                    quarter(st, Q3{}, l2, std::integral_constant<int, M2>{}, std::integral_constant<int, NEXT2 ? L - M2 : 0>{}, NoSync{});
+                };
+                const uint32_t ahead = t.k_tiles >= 2 ? t.k_tiles - 2 : 0u;   // slices that request slice kt+2
+                for (uint32_t kt = 0; kt < ahead; ++kt) slice(kt, std::true_type{}, std::true_type{});
+                if (t.k_tiles >= 2) slice(t.k_tiles - 2, std::true_type{}, std::false_type{});
+                slice(t.k_tiles - 1, std::false_type{}, std::false_type{});
+            } else if constexpr (AHEAD2) {
                 static_assert(LA + LB <= kPerQuarter, "the loads of a slice fit behind the matrix instructions of one quarter");
                 constexpr int N0 = spread_count(0), N1 = spread_count(1), N2 = spread_count(2), N3 = spread_count(3);
                 // Slice 0 was requested by begin(). Every wavefront has left the previous tile's epilogue,
@@ -621,9 +693,16 @@ struct Gemm16 {
                     const char* st = smem + stage_of(t, kt) * kStage;
                     read_fragments(st, 0);
                     const SliceLoads l1 = NEXT ? loads_of(kt + 1) : SliceLoads{};
-                    quarter(st, Q0{}, l1, std::integral_constant<int, N0>{}, std::integral_constant<int, NEXT ? N1 : 0>{});
-                    quarter(st, Q1{}, l1, std::integral_constant<int, N0 + N1>{}, std::integral_constant<int, NEXT ? N2 : 0>{});
-                    quarter(st, Q2{}, l1, std::integral_constant<int, N0 + N1 + N2>{}, std::integral_constant<int, NEXT ? N3 : 0>{});
+                    quarter(st, Q0{}, l1, std::integral_constant<int, N0>{}, std::integral_constant<int, NEXT ? N1 : 0>{}, NoSync{});
+                    quarter(st, Q1{}, l1, std::integral_constant<int, N0 + N1>{}, std::integral_constant<int, NEXT ? N2 : 0>{}, NoSync{});
+                    if constexpr (kEarlyFirst) {
+                        const SliceLoads l2 = NEXT2 ? loads_of(kt + 2) : SliceLoads{};
+                        quarter(st, Q2{}, l2, std::integral_constant<int, 0>{}, std::integral_constant<int, NEXT2 ? N0 : 0>{},
+                                std::integral_constant<int, NEXT2 ? kReleaseAt : -1>{});
+                        quarter(st, Q3{}, l2, std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}, NoSync{});
+                        return;
+                    }
+                    quarter(st, Q2{}, l1, std::integral_constant<int, N0 + N1 + N2>{}, std::integral_constant<int, NEXT ? N3 : 0>{}, NoSync{});
                     if constexpr (NEXT2) {
                         // this wavefront's last reads of the stage have returned; once that holds for every
                         // wavefront the stage takes slice kt+2
@@ -631,7 +710,7 @@ struct Gemm16 {
                         asm volatile("s_barrier" ::: "memory");
                     }
                     const SliceLoads l2 = NEXT2 ? loads_of(kt + 2) : SliceLoads{};
-                    quarter(st, Q3{}, l2, std::integral_constant<int, 0>{}, std::integral_constant<int, NEXT2 ? N0 : 0>{});
+                    quarter(st, Q3{}, l2, std::integral_constant<int, 0>{}, std::integral_constant<int, NEXT2 ? N0 : 0>{}, NoSync{});
                 };
                 const uint32_t ahead = t.k_tiles >= 2 ? t.k_tiles - 2 : 0u;   // slices that request slice kt+2
                 for (uint32_t kt = 0; kt < ahead; ++kt) slice(kt, std::true_type{}, std::true_type{});
@@ -660,7 +739,7 @@ struct Gemm16 {
                         constexpr int q = decltype(q_tag)::value;
                         constexpr int left = LA + LB - q * kPerQuarter;
                         constexpr int count = !decltype(loads_tag)::value || left <= 0 ? 0 : (left < kPerQuarter ? left : kPerQuarter);
-                        quarter(st, q_tag, l, std::integral_constant<int, q * kPerQuarter>{}, std::integral_constant<int, count>{});
+                        quarter(st, q_tag, l, std::integral_constant<int, q * kPerQuarter>{}, std::integral_constant<int, count>{}, NoSync{});
                     });
                 };
                 const uint32_t ahead = t.k_tiles >= uint32_t(STAGES - 1) ? t.k_tiles - (STAGES - 1) : 0u;   // slices that request a later one
