@@ -65,6 +65,7 @@ class Workload:
     w_std: float
     zipf_s: float = 0.0          # > 0: per-expert logit bias from a Zipf ranking, injected through the data
     hot_ratio: float = 0.0       # target load of the hottest expert relative to the mean
+    forced_rows: tuple = ()      # non-empty (top-1 only): expert e is routed exactly forced_rows[e] tokens
     note: str = ""
 
 
@@ -85,6 +86,10 @@ WORKLOADS = {
                            note="S=8192 H=4096 I=14336 E=8 top-2 cf=1.25 bf16"),
     "fine_e256_top8": Workload("fine_e256_top8", _cfg(4096, 7168, 2048, 256, 8, 1.0, 2), 1.0, 0.01,
                                note="S=4096 H=7168 I=2048 E=256 top-8 cf=1.0 bf16"),
+    # the expert projections of mixtral_e8 (16 384 rows over 8 experts) with every 256-row block full
+    "mixtral_full_blocks": Workload("mixtral_full_blocks", _cfg(16384, 4096, 14336, 8, 1, 1.0, 2), 1.0, 0.01,
+                                    forced_rows=(2048,) * 8,
+                                    note="S=16384 H=4096 I=14336 E=8 top-1 cf=1.0 bf16, 2048 tokens routed to every expert"),
 }
 
 
@@ -92,7 +97,7 @@ def scaled(workload: Workload, **overrides) -> Workload:
     """The same data recipe on different sizes (for parity tests the checker can finish quickly)."""
     cfg = KleosConfig(**{**workload.config.__dict__, **overrides})
     return Workload(workload.name + "_scaled", cfg, workload.x_std, workload.w_std, workload.zipf_s,
-                    workload.hot_ratio, workload.note)
+                    workload.hot_ratio, workload.forced_rows, workload.note)
 
 
 def _torch_dtype(derived: DerivedConfig):
@@ -136,6 +141,8 @@ def make_inputs(workload: Workload, seed: int = 0, device: str = "cuda", portabl
 
     if workload.zipf_s > 0:
         _inject_zipf_bias(buf, d, workload, seed)
+    if workload.forced_rows:
+        _force_routing(buf, d, workload, seed)
     if d.keys.torch_dtype == 1:
         _round_tf32_(buf)   # main.cu:59-62 converts every input to Element, here tfloat32_t
     return buf, d
@@ -147,6 +154,24 @@ def _round_tf32_(buf) -> None:
     u = buf.view(torch.int32)
     finite = (u & 0x7F800000) != 0x7F800000
     u.copy_(torch.where(finite, u + 0x0FFF + ((u >> 13) & 1), u) & ~0x1FFF)
+
+
+def _force_routing(buf, d: DerivedConfig, w: Workload, seed: int) -> None:
+    """Routing decided by the data (top-1): the first E hidden features of a token are one-hot in the
+    expert it is meant for, and the gate weights read them back (Wg[e, :E] = unit vector e, the other
+    gate weights damped), so that expert e receives exactly forced_rows[e] tokens, in a shuffled order."""
+    import torch
+
+    S, H, E = d.S, d.H, d.E
+    assert d.k == 1 and len(w.forced_rows) == E and sum(w.forced_rows) == S
+    x = buf[d.off_x:d.off_x + S * H].view(S, H)
+    wg = buf[d.off_gate_w:d.off_gate_w + E * H].view(E, H)
+    owner = np.repeat(np.arange(E), w.forced_rows)[portable_permutation(seed, 2000, S)]
+    owner = torch.from_numpy(owner.astype(np.int64)).to(buf.device)
+    x[:, :E] = 0.0
+    x[torch.arange(S, device=buf.device), owner] = 8.0
+    wg[:, :E] = torch.eye(E, dtype=buf.dtype, device=buf.device)
+    wg[:, E:] *= 0.25
 
 
 def _inject_zipf_bias(buf, d: DerivedConfig, w: Workload, seed: int) -> float:

@@ -33,6 +33,7 @@ def test_parse_shipped_config_keys():
     ("headline_e64_zipf", 8192, 64, 256, 256, 8192 * 2048 + 64 * 2048 + 2 * 64 * 2048 * 2048 + 64 * 4096),
     ("mixtral_e8", 8192, 64, 2560, 2560, 8192 * 4096 + 64 * 4096 + 2 * 8 * 14336 * 4096 + 8 * (14336 + 4096)),
     ("fine_e256_top8", 4096, 256, 128, 128, 4096 * 7168 + 256 * 7168 + 2 * 256 * 2048 * 7168 + 256 * (2048 + 7168)),
+    ("mixtral_full_blocks", 16384, 64, 2048, 2048, 16384 * 4096 + 64 * 4096 + 2 * 8 * 14336 * 4096 + 8 * (14336 + 4096)),
 ])
 def test_workload_configs_derive_the_reference_constants(name, S, PX, EC, pEC, in_elems):
     cfg = ka.KleosConfig.from_json_file(os.path.join(CONFIG_DIR, name + ".json"))

@@ -42,3 +42,19 @@ def test_oracle_reproduces_the_fixture(tiny, oracle):
     assert np.abs(out["logits"] - g["logits"]).max() < 1e-6
     assert rel_fro(out["moe_out"], g["moe_out"]) < 1e-6
     assert np.abs(out["gate_out"][:, :c.E] - g["gate_out"]).max() < 1e-6
+
+
+def test_forced_routing_gives_every_expert_its_rows(oracle):
+    """A workload with `forced_rows` routes exactly that many tokens to each expert (top-1, decided by
+    one-hot input features the gate weights read back): checked with the oracle's gate and routing."""
+    rows = (10, 50, 32, 0, 64, 1, 99, 128)
+    w = synth.Workload("forced_small", synth._cfg(sum(rows), 128, 256, 8, 1, 4.0, 0), 1.0, 0.05, forced_rows=rows)
+    iP, d = synth.make_inputs(w, seed=3, device="cpu")
+    c = oracle.cfg_from_keys(w.config)
+    out = oracle.forward(c, iP.numpy())
+    np.testing.assert_array_equal(out["expert_count"], np.array(rows))
+    assert (out["topk_slot"] >= 0).all()                       # capacity 4 x the mean: nothing dropped
+    iP2, _ = synth.make_inputs(w, seed=4, device="cpu")        # another seed: another order, the same counts
+    out2 = oracle.forward(c, iP2.numpy())
+    np.testing.assert_array_equal(out2["expert_count"], np.array(rows))
+    assert not np.array_equal(out["topk_expert"], out2["topk_expert"])

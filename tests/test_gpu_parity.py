@@ -684,6 +684,24 @@ def test_fine_e256_top8_full_size(mode):
     assert v["expert_count"].astype(np.int64).sum() == c.S * c.k
 
 
+@pytest.mark.parametrize("mode", MODES, ids=MODE_IDS)
+def test_forced_full_row_blocks_at_reduced_width(mode):
+    """The recipe of the mixtral_full_blocks workload (top-1, every expert routed exactly the rows of
+    its capacity, all row blocks full) on narrower projections: 8 experts x 1 024 rows, so the 256-row
+    tiles of the variant for large experts, no ragged block, nothing dropped."""
+    full = synth.WORKLOADS["mixtral_full_blocks"]
+    w = synth.Workload("full_blocks_small", synth._cfg(8192, 512, 1024, 8, 1, 1.0, 2), full.x_std, 0.03,
+                       forced_rows=(1024,) * 8)
+    iP, d = synth.make_inputs(w, seed=5, device="cuda")
+    c = moe_ref.cfg_from_keys(w.config)
+    assert c.EC == 1024
+    mask = np.zeros(c.S, np.uint8)
+    mask[np.random.default_rng(5).choice(c.S, size=256, replace=False)] = 1
+    d, v, moe_out, err = check_against_oracle(c, w.config, _out_to_np(c, iP), mode, token_mask=mask)
+    np.testing.assert_array_equal(v["expert_count"], np.full(8, 1024))
+    assert (v["topk_slot"] >= 0).all()
+
+
 @pytest.mark.parametrize("name,schedule", [("headline_e64_zipf", ka.SCHEDULE_STATIC), ("headline_e64_zipf", ka.SCHEDULE_DYNAMIC),
                                            ("balanced_e16", ka.SCHEDULE_AUTO), ("fine_e256_top8", ka.SCHEDULE_AUTO)],
                          ids=["headline-static", "headline-dynamic", "balanced_e16", "fine_e256_top8"])
