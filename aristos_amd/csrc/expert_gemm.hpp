@@ -132,7 +132,13 @@ constexpr int kEpiloguePanelRows = 32;
 // any XCD, and nothing then has to write a whole L2 back before it may tell them so. It also pays
 // by itself where a launch writes far more output than the L2 holds (256-expert top-8 shape: 3.03
 // against 3.11 ms per forward); neutral on the other shapes measured.
-template <typename E, int WM, int WN, int WAVES_N, int ACT>
+// STREAM_OUT adds the non-temporal hint: the rows pass through the L2 without staying there. For
+// layers of many small experts, whose intermediate and output rows are many times the L2 and are
+// read long after they were written (256-expert top-8 shape: 2 865 against 2 950 us per forward with
+// both outputs streamed, 2 913 with the intermediate rows alone, 2 953 with the output rows alone);
+// where the rows are read back soon, from the L2 that took them, it costs (64-expert shape 293
+// against 287 us, 16-expert shape 154 against 146 us).
+template <typename E, int WM, int WN, int WAVES_N, int ACT, bool STREAM_OUT>
 __device__ __forceinline__ void epilogue16_act(const TileOut& t, f32x16 (&acc)[WN / 32][WM / 32], char* stage_mem,
                                                const char* bias_mem) {
     typedef typename Elem16<E>::vec4 vec4;
@@ -169,7 +175,7 @@ __device__ __forceinline__ void epilogue16_act(const TileOut& t, f32x16 (&acc)[W
                 const u32x4 v = load16(stg + r * 128 + ((c ^ ((r >> 1) & 7)) << 4));
                 const uint32_t m = wm * WM + mi * 32 + r, n = wn * WN + pn * 64 + c * 8;
                 if (m < t.m_valid && n < t.n_valid) {
-                    constexpr int kAgentScope = 16;   // sc1
+                    constexpr int kAgentScope = STREAM_OUT ? 16 + 2 : 16;   // sc1 (+ nt)
                     // (a tile's rows lie within 2 GiB of its first element: 256 rows of at most 2^22 bytes)
                     __builtin_amdgcn_raw_buffer_store_b128(v, coherent_rows(t.c_base), int((size_t(m) * t.ldc + n) * sizeof(E)), 0,
                                                            kAgentScope);
@@ -178,18 +184,18 @@ __device__ __forceinline__ void epilogue16_act(const TileOut& t, f32x16 (&acc)[W
         }
     }
 }
-template <typename E, int WM, int WN, int WAVES_N>
+template <typename E, int WM, int WN, int WAVES_N, bool STREAM_OUT>
 __device__ __forceinline__ void epilogue16(const TileOut& t, f32x16 (&acc)[WN / 32][WM / 32], char* stage_mem,
                                            const char* bias_mem) {
-    if (t.act == 0) epilogue16_act<E, WM, WN, WAVES_N, 0>(t, acc, stage_mem, bias_mem);
-    else if (t.act == 1) epilogue16_act<E, WM, WN, WAVES_N, 1>(t, acc, stage_mem, bias_mem);
-    else epilogue16_act<E, WM, WN, WAVES_N, 2>(t, acc, stage_mem, bias_mem);
+    if (t.act == 0) epilogue16_act<E, WM, WN, WAVES_N, 0, STREAM_OUT>(t, acc, stage_mem, bias_mem);
+    else if (t.act == 1) epilogue16_act<E, WM, WN, WAVES_N, 1, STREAM_OUT>(t, acc, stage_mem, bias_mem);
+    else epilogue16_act<E, WM, WN, WAVES_N, 2, STREAM_OUT>(t, acc, stage_mem, bias_mem);
 }
 
 // The same epilogue for accumulators of 16 x 16 matrix-core tiles: acc[ni][mi][v] is output column
 // n = wn*WN + ni*16 + 4*(lane/16) + v of output row m = wm*WM + mi*16 + lane%16 - again 4 consecutive
 // columns per lane and tile, so the panels, their LDS layout and the stores are the ones above.
-template <typename E, int WM, int WN, int WAVES_N, int ACT>
+template <typename E, int WM, int WN, int WAVES_N, int ACT, bool STREAM_OUT>
 __device__ __forceinline__ void epilogue16_act(const TileOut& t, f32x4 (&acc)[WN / 16][WM / 16], char* stage_mem,
                                                const char* bias_mem) {
     typedef typename Elem16<E>::vec4 vec4;
@@ -226,7 +232,7 @@ __device__ __forceinline__ void epilogue16_act(const TileOut& t, f32x4 (&acc)[WN
                 const u32x4 v = load16(stg + r * 128 + ((c ^ ((r >> 1) & 7)) << 4));
                 const uint32_t m = wm * WM + pm * 32 + r, n = wn * WN + pn * 64 + c * 8;
                 if (m < t.m_valid && n < t.n_valid) {
-                    constexpr int kAgentScope = 16;   // sc1
+                    constexpr int kAgentScope = STREAM_OUT ? 16 + 2 : 16;   // sc1 (+ nt)
                     __builtin_amdgcn_raw_buffer_store_b128(v, coherent_rows(t.c_base), int((size_t(m) * t.ldc + n) * sizeof(E)), 0,
                                                            kAgentScope);
                 }
@@ -234,12 +240,12 @@ __device__ __forceinline__ void epilogue16_act(const TileOut& t, f32x4 (&acc)[WN
         }
     }
 }
-template <typename E, int WM, int WN, int WAVES_N>
+template <typename E, int WM, int WN, int WAVES_N, bool STREAM_OUT>
 __device__ __forceinline__ void epilogue16(const TileOut& t, f32x4 (&acc)[WN / 16][WM / 16], char* stage_mem,
                                            const char* bias_mem) {
-    if (t.act == 0) epilogue16_act<E, WM, WN, WAVES_N, 0>(t, acc, stage_mem, bias_mem);
-    else if (t.act == 1) epilogue16_act<E, WM, WN, WAVES_N, 1>(t, acc, stage_mem, bias_mem);
-    else epilogue16_act<E, WM, WN, WAVES_N, 2>(t, acc, stage_mem, bias_mem);
+    if (t.act == 0) epilogue16_act<E, WM, WN, WAVES_N, 0, STREAM_OUT>(t, acc, stage_mem, bias_mem);
+    else if (t.act == 1) epilogue16_act<E, WM, WN, WAVES_N, 1, STREAM_OUT>(t, acc, stage_mem, bias_mem);
+    else epilogue16_act<E, WM, WN, WAVES_N, 2, STREAM_OUT>(t, acc, stage_mem, bias_mem);
 }
 
 // f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>), in this order.
@@ -289,8 +295,9 @@ __device__ __forceinline__ void static_for(F&& f) {
 // half slices to land (16-expert shape 146 against 150 us, 64-expert shape 284 against 287 us; the
 // 8-expert shape loses, 3 177 against 3 115 us: its loads, bunched into half a slice, hold up the
 // matrix instructions behind them).
+// STREAM_OUT: the output rows are stored with the non-temporal hint (see the epilogue above).
 template <typename E, int BM, int BN, int WAVES_M, int WAVES_N, int BK, int STAGES, bool STREAM_B, bool AHEAD2, int SPREAD = 0, int MI = 32,
-          int RELEASE = 0>
+          int RELEASE = 0, bool STREAM_OUT = false>
 struct Gemm16 {
     typedef typename Elem16<E>::vec8 vec8;
     typedef typename Elem16<E>::vec4 vec4;
@@ -826,7 +833,7 @@ struct Gemm16 {
     static __device__ __forceinline__ void finish(const Tile& t, Acc& acc, char* smem) {
         if (rows_absent(t, __builtin_amdgcn_readfirstlane(int(local_tid() >> 6)) / WAVES_N)) return;   // nothing of this wavefront's is stored
         const TileOut out{t.c_base, t.ldc, t.m_valid, t.n_valid, t.act};
-        epilogue16<E, WM, WN, WAVES_N>(out, acc, smem + last_stage(t) * kStage, smem + kBiasOffset + t.bias_slot * kBiasBytes);
+        epilogue16<E, WM, WN, WAVES_N, STREAM_OUT>(out, acc, smem + last_stage(t) * kStage, smem + kBiasOffset + t.bias_slot * kBiasBytes);
     }
 };
 

@@ -82,6 +82,9 @@ constexpr int kXcds = 8;
 #ifndef KLEOS_TUNE_MI_V0
 #define KLEOS_TUNE_MI_V0 16        // the same for variant 0 (switchable apart: its tiles are the ones bound by their loads)
 #endif
+#ifndef KLEOS_TUNE_V1_STREAM_OUT
+#define KLEOS_TUNE_V1_STREAM_OUT 1 // variant 1 (many small experts) stores its intermediate and output rows non-temporally
+#endif
 #ifndef KLEOS_TUNE_V0_RELEASE
 #define KLEOS_TUNE_V0_RELEASE 1    // where variant 0 frees a slice's stage and issues the loads behind it (Gemm16's RELEASE)
 #endif
@@ -90,7 +93,7 @@ constexpr int kXcds = 8;
 #endif
 template <typename E, int V>
 using GemmCfg = std::conditional_t<V == 0, Gemm16<E, 256, 256, 4, 2, 64, 2, true, true, KLEOS_TUNE_V0_SPREAD, KLEOS_TUNE_MI_V0, KLEOS_TUNE_V0_RELEASE>,
-                std::conditional_t<V == 1, Gemm16<E, 128, 256, 2, 4, 64, 3, true, false, 0, KLEOS_TUNE_MI>,
+                std::conditional_t<V == 1, Gemm16<E, 128, 256, 2, 4, 64, 3, true, false, 0, KLEOS_TUNE_MI, 0, (KLEOS_TUNE_V1_STREAM_OUT != 0)>,
                                    Gemm16<E, 256, 256, 2, 4, 64, 2, false, (KLEOS_TUNE_V2_SPREAD >= 0), (KLEOS_TUNE_V2_SPREAD >= 0 ? KLEOS_TUNE_V2_SPREAD : 0), KLEOS_TUNE_MI,
                                           KLEOS_TUNE_V2_RELEASE>>>;
 // Layers of variant 2 mix two tile heights inside one launch: the last row block of an expert, when
