@@ -82,7 +82,7 @@ ArenaLayout layout_arena(const kleos_config_t& c, uint32_t n_tiles, uint32_t n_s
     L.tile_count = take(size_t(n_tiles) * E * 4);
     L.slot_token = take(E * R * 4);
     L.h1 = take(E * R * size_t(c.I) * c.elem_bytes);
-    L.y = take(E * R * size_t(c.H) * c.elem_bytes);
+    L.y = take(E * y_expert_elems(uint32_t(R), c.H, c.elem_bytes) * c.elem_bytes);
     L.gate_partial = take(size_t(gate_splits) * S * c.PX * 4);
     // one expert: gate weights (zeros) and a gate output of the library's own, for callers that pack the
     // dense-FFN way, without either (kleos_moe_forward_dense)
@@ -710,7 +710,7 @@ extern "C" int kleos_measure_throughput_output(uint32_t trials, float* median_ms
     size_t off = 0;
     auto take = [&](size_t bytes) { size_t o = off; off = align_up(off + bytes, 256); return o; };
     const size_t o_x = take(M * H * eb), o_wu = take(I * H * eb), o_wd = take(H * I * eb), o_bu = take(I * eb),
-                 o_bd = take(H * eb), o_h1 = take(M * I * eb), o_y = take(M * H * eb), o_cnt = take(4),
+                 o_bd = take(H * eb), o_h1 = take(M * I * eb), o_y = take(y_expert_elems(uint32_t(M), cfg.H, cfg.elem_bytes) * eb), o_cnt = take(4),
                  o_tok = take(M * 4);
     char* buf = nullptr;
     KLEOS_HIP(hipMalloc(reinterpret_cast<void**>(&buf), off));
@@ -748,7 +748,15 @@ extern "C" int kleos_measure_throughput_output(uint32_t trials, float* median_ms
         std::sort(ms.begin(), ms.end());
         *median_ms = ms[trials / 2];                          // throughput.cuh:166 (findMedian)
         *throughput = *median_ms > 0.f ? 1.0f / *median_ms : 0.f;
-        if (y_bytes) KLEOS_HIP(hipMemcpy(y_host, buf + o_y, y_bytes, hipMemcpyDeviceToHost));
+        if (y_bytes) {
+            // the caller gets y[pEC, H] row by row, whatever the layout the kernels keep it in
+            std::vector<char> dev_y(y_expert_elems(uint32_t(M), cfg.H, cfg.elem_bytes) * eb), rows(M * H * eb);
+            KLEOS_HIP(hipMemcpy(dev_y.data(), buf + o_y, dev_y.size(), hipMemcpyDeviceToHost));
+            for (size_t m = 0; m < M; ++m)
+                for (size_t n = 0; n < H; ++n)
+                    std::memcpy(&rows[(m * H + n) * eb], &dev_y[y_offset(0, uint32_t(m), uint32_t(n), uint32_t(M), cfg.H, cfg.elem_bytes) * eb], eb);
+            std::memcpy(y_host, rows.data(), y_bytes);
+        }
         return KLEOS_OK;
     };
     rc = body();

@@ -49,6 +49,11 @@ __device__ __forceinline__ void combine_tokens_inline(const LayerParams& p, uint
     const uint32_t H = p.H, k = p.k;
     const T* y = static_cast<const T*>(p.y);
     const uint32_t col_stride = kWave * kPer;
+    // byte offset of column `col` inside a row of y (a lane's 16 bytes never straddle two pieces)
+    auto row_offset = [&](uint32_t col) {
+        if constexpr (sizeof(T) == 2) return uint32_t((size_t(col / kOutPiece) * p.cap_rows * kOutPiece + col % kOutPiece) * sizeof(T));
+        else return uint32_t(col * sizeof(T));
+    };
 
     if (first >= p.S) return;
     CombineRoute<KMAX> cur = combine_route<KMAX>(p, first);
@@ -67,8 +72,7 @@ __device__ __forceinline__ void combine_tokens_inline(const LayerParams& p, uint
             // (indices clamped to their tables: no value they could hold leaves the y buffer)
             const uint32_t e = uint32_t(cur.expert[r]) < p.E ? uint32_t(cur.expert[r]) : p.E - 1;
             const uint32_t sl = uint32_t(cur.slot[r]) < p.cap_rows ? uint32_t(cur.slot[r]) : p.cap_rows - 1;
-            const size_t row = on[r] ? size_t(e) * p.cap_rows + sl : 0;
-            rows[r] = coherent_rows(y + row * H);
+            rows[r] = coherent_rows(y + (on[r] ? y_offset(e, sl, 0, p.cap_rows, H, sizeof(T)) : 0));
             scale[r] = elem_to_float(float_to_elem<T>(cur.prob[r]));
         }
         T* out = static_cast<T*>(p.moe_out) + size_t(token) * H;
@@ -78,7 +82,7 @@ __device__ __forceinline__ void combine_tokens_inline(const LayerParams& p, uint
             for (int c = 0; c < CH; ++c)
 #pragma unroll
                 for (int r = 0; r < KMAX; ++r)
-                    if (on[r] && c0 + c * col_stride < H) v[c][r] = load16_coherent(rows[r], (c0 + c * col_stride) * sizeof(T));
+                    if (on[r] && c0 + c * col_stride < H) v[c][r] = load16_coherent(rows[r], row_offset(c0 + c * col_stride));
 #pragma unroll
             for (int c = 0; c < CH; ++c) {
                 if (c0 + c * col_stride >= H) break;
@@ -131,7 +135,8 @@ __device__ __forceinline__ void combine_tokens_generic(const LayerParams& p, uin
                 uint32_t e = uint32_t(load_coherent(p.topk_expert + size_t(token) * k + r));
                 if (e >= p.E || uint32_t(slot) >= p.cap_rows) continue;
                 const float scale = elem_to_float(float_to_elem<T>(load_coherent(p.topk_prob + size_t(token) * k + r)));
-                const u32x4 raw = load16_coherent(coherent_rows(y + (size_t(e) * p.cap_rows + uint32_t(slot)) * H), c0 * sizeof(T));
+                const u32x4 raw = load16_coherent(coherent_rows(y + y_offset(e, uint32_t(slot), 0, p.cap_rows, H, sizeof(T))),
+                                                  uint32_t((y_offset(0, 0, c0, p.cap_rows, H, sizeof(T))) * sizeof(T)));
                 T vals[kPer];
                 __builtin_memcpy(vals, &raw, 16);
 #pragma unroll

@@ -330,7 +330,13 @@ __device__ __forceinline__ TileOperands<T> tile_operands(const LayerParams& p, c
         o.c = static_cast<T*>(p.h1) + row_base * p.I + col0; o.ldc = p.I; o.act = p.act;
     } else {
         o.a = static_cast<const T*>(p.h1) + row_base * p.I; o.idx = nullptr; o.lda = p.I;
-        o.c = static_cast<T*>(p.y) + row_base * p.H + col0; o.ldc = p.H; o.act = 2;
+        o.act = 2;
+        if constexpr (sizeof(T) == 2) {   // the tile's piece of y: cap_rows rows of kOutPiece columns
+            static_assert(BN == int(kOutPiece));
+            o.c = static_cast<T*>(p.y) + y_offset(t.e, row0, col0, p.cap_rows, p.H, sizeof(T)); o.ldc = kOutPiece;
+        } else {
+            o.c = static_cast<T*>(p.y) + row_base * p.H + col0; o.ldc = p.H;
+        }
     }
     return o;
 }

@@ -182,6 +182,8 @@ CASES = [
     (256, 192, 64, 512, 6, 2.0, 1, 1, 2, 0.1),     # E = 512, cf = 2, gelu + biases
     (256, 64, 64, 384, 4, 1.0, 1, 0, 0, 0.0),      # fp32, E = 384
     (256, 1088, 64, 320, 4, 1.0, 1, 0, 2, 0.0),    # E = 320 over a long hidden dimension: batched and single K steps
+    (128, 320, 64, 96, 40, 1.0, 1, 0, 2, 0.0),     # 40 picks per token (the combine that re-reads its routing) over output rows of two 256-column pieces
+    (256, 576, 128, 16, 2, 1.0, 1, 1, 3, 0.1),     # fp16, output rows of two pieces and a quarter
 ]
 
 
